@@ -30,9 +30,12 @@ sys.path.insert(0, str(ROOT))
 
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size) measured
-# with rocprofv3 --pmc for the workloads listed; the summaries are under profiles/.
-MEASURED_TRAFFIC = {("f16", "NN", 8192, 8192, 8192): 1744771072}
+# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size) come from
+# rocprofv3 --pmc runs, not from this process: profiles/hbm_traffic.txt lists them, one workload per line,
+# with the summary file that documents the run.
+TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic.txt"
+# Untimed launches in front of --warmup: the clocks of an idle part take ~0.1 s of this kernel to ramp.
+RAMP_SECONDS = 0.3
 DT = {"f32": 0, "f16": 1, "bf16": 2}
 ESIZE = {"f32": 4, "f16": 2, "bf16": 2}
 
@@ -55,6 +58,9 @@ def parse_args():
     p.add_argument("--n", type=int, default=0, help="N if different from --size (skinny shapes)")
     p.add_argument("--beta", type=float, default=0.0)
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    p.add_argument("--no-ramp", action="store_true", help="skip the untimed clock ramp in front of --warmup")
+    p.add_argument("--no-configs", action="store_true",
+                   help="skip the MLP / LSTM / GPT-layer passes that fill the `configs` block")
     p.add_argument("--cpu-panel", type=int, default=8192,
                    help="columns of the product that the CPU baseline computes")
     p.add_argument("--report", default="", help="write the sweep results to this JSON file")
@@ -90,12 +96,20 @@ class Harness:
         t.cuda.synchronize()
         return A, B, C, a_rows, b_rows
 
-    def time_gemm(self, dtype, layout, m, n, k, steps, warmup, beta=0.0):
+    def time_gemm(self, dtype, layout, m, n, k, steps, warmup, beta=0.0, ramp_seconds=0.0):
         A, B, C, lda, ldb = self.operands(dtype, layout, m, n, k)
         op_a, op_b = int(layout[0] == "T"), int(layout[1] == "T")
         lib, ctx = self.lib, self.ctx
         args = (ctx, DT[dtype], op_a, op_b, m, n, k, c_void_p(A.data_ptr()), lda,
                 c_void_p(B.data_ptr()), ldb, beta, c_void_p(C.data_ptr()), m)
+        # Time-bounded, untimed ramp: the same launches until ramp_seconds have passed, whatever --warmup is.
+        self.ramp_launches = 0
+        t_end = time.perf_counter() + ramp_seconds
+        while ramp_seconds > 0 and time.perf_counter() < t_end:
+            for _ in range(8):
+                lib.call("ginn_hip_gemm", *args)
+            lib.call("ginn_hip_sync", ctx)
+            self.ramp_launches += 8
         for _ in range(warmup):
             lib.call("ginn_hip_gemm", *args)
         lib.call("ginn_hip_sync", ctx)
@@ -402,6 +416,38 @@ def cpu_baseline(m, k, panel, dtype):
     }
 
 
+def measured_traffic(dtype, layout, m, n, k):
+    """(bytes per launch, source) from profiles/hbm_traffic.txt, or (None, None)."""
+    if not TRAFFIC_FILE.exists():
+        return None, None
+    for line in TRAFFIC_FILE.read_text().splitlines():
+        f = line.split()
+        if len(f) >= 7 and not line.startswith("#") and f[:5] == [dtype, layout, str(m), str(n), str(k)]:
+            return int(f[5]), f[6]
+    return None, None
+
+
+def other_configs(cpu):
+    """The graph-level configurations of the build target, a few passes each, outside the headline's timed
+    region: GPU ms per fwd+bwd pass through the frozen level executor, and the CPU oracle on one thread."""
+    out = {}
+    g = bench_gpt(4, cpu, executor=6)
+    out["gpt_ms"], out["gpt_tflops"] = g["gpu_ms"], g["tflops"]
+    if cpu:
+        out["gpt_cpu_ms"] = g["cpu_ms"]
+    r = bench_mlp(20, cpu, executor=6)
+    out["mlp_ms"] = r["gpu_ms"]
+    if cpu:
+        out["mlp_cpu_ms"] = r["cpu_ms"]
+    r = bench_lstm(4, cpu, mode=23, gather=True)
+    out["lstm_ms"] = r["gpu_ms"]
+    if cpu:
+        out["lstm_cpu_ms"] = r["cpu_ms"]
+    out["note"] = ("fwd+bwd per pass: min-GPT layer bf16 (d768 h12 T512 B8 ff3072 V8192), MLP fp32 b64 784-512-512-10, "
+                   "autobatched LSTM fp32 256 seqs; cpu = numpy fp32 oracle on 1 thread")
+    return out
+
+
 def main():
     a = parse_args()
     if a.gpus != 1:
@@ -485,7 +531,9 @@ def main():
             Path(a.report).parent.mkdir(parents=True, exist_ok=True)
             Path(a.report).write_text(json.dumps(results, indent=1))
 
-    wall, kernel_ms, _ = h.time_gemm(a.dtype, a.layout, m, n, k, a.steps, a.warmup, a.beta)
+    wall, kernel_ms, _ = h.time_gemm(a.dtype, a.layout, m, n, k, a.steps, a.warmup, a.beta,
+                                     ramp_seconds=0.0 if a.no_ramp else RAMP_SECONDS)
+    traffic, traffic_source = measured_traffic(a.dtype, a.layout, m, n, k) if a.beta == 0 else (None, None)
     flops = 2.0 * m * n * k
     value = flops * a.steps / wall / 1e12
     achieved = flops / (kernel_ms * 1e-3) / 1e12
@@ -497,6 +545,7 @@ def main():
         "n_gpus": 1,
         "steps": a.steps,
         "warmup": a.warmup,
+        "ramp_launches": h.ramp_launches,
         "ms_per_step": round(wall / a.steps * 1e3, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -512,12 +561,15 @@ def main():
             "peak": PEAK_TFLOPS[a.dtype],
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_TFLOPS[a.dtype], 4),
-            "traffic": MEASURED_TRAFFIC.get((a.dtype, a.layout, m, n, k)) if a.beta == 0 else None,
+            "traffic": traffic,
+            "traffic_source": traffic_source,
             "kernel_ms": round(kernel_ms, 4),
         },
     }
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(m, k, min(a.cpu_panel, n), a.dtype)
+    if not a.no_configs:
+        line["configs"] = other_configs(not a.no_cpu)
     print(json.dumps(line), flush=True)
 
 

@@ -40,6 +40,7 @@ PROTOTYPES = {
     "ginn_hip_arena_destroy": (c_int, [c_void_p]),
     "ginn_hip_arena_alloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "ginn_hip_arena_clear": (c_int, [c_void_p]),
+    "ginn_hip_arena_set_alignment": (c_int, [c_void_p, c_size_t]),
     "ginn_hip_arena_used": (c_int, [c_void_p, POINTER(c_size_t)]),
     "ginn_hip_arena_size": (c_int, [c_void_p, POINTER(c_size_t)]),
     "ginn_hip_gemm": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,

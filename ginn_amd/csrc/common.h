@@ -79,6 +79,7 @@ struct ginn_hip_arena {
   char* base = nullptr;
   size_t size = 0;
   size_t used = 0;
+  size_t alignment = 1;  // start of every block; 1 = byte-exact bump
 };
 
 namespace ginn_hip {

@@ -281,16 +281,26 @@ int ginn_hip_arena_destroy(ginn_hip_arena* arena) {
 
 int ginn_hip_arena_alloc(ginn_hip_arena* arena, size_t bytes, void** ptr) {
   GH_CHECK_ARG(arena && ptr, "ginn_hip_arena_alloc: NULL argument");
-  const size_t aligned = (bytes + 255) & ~size_t(255);
-  // Strict '<' as in PreallocGpuDevice::alloc (ginn/dev.h:238-241).
-  if (!(arena->used + aligned < arena->size)) {
+  // Byte-exact bump with the strict '<' of PreallocGpuDevice::alloc
+  // (ginn/dev.h:238-241) unless the caller asked for aligned blocks.
+  const size_t al = arena->alignment;
+  const size_t start = al > 1 ? (arena->used + al - 1) / al * al : arena->used;
+  if (!(start + bytes < arena->size)) {
     *ptr = nullptr;
     return fail(kOutOfMemory,
                 "Prealloc device out of memory! Used: %zu Attempted to allocate: %zu",
                 arena->used, bytes);
   }
-  *ptr = arena->base + arena->used;
-  arena->used += aligned;
+  *ptr = arena->base + start;
+  arena->used = start + bytes;
+  return kOk;
+}
+
+int ginn_hip_arena_set_alignment(ginn_hip_arena* arena, size_t alignment) {
+  GH_CHECK_ARG(arena, "ginn_hip_arena_set_alignment: arena is NULL");
+  GH_CHECK_ARG(alignment >= 1 && alignment <= 4096 && (alignment & (alignment - 1)) == 0,
+               "ginn_hip_arena_set_alignment: %zu is not a power of two in 1..4096", alignment);
+  arena->alignment = alignment;
   return kOk;
 }
 

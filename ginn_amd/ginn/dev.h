@@ -2,9 +2,9 @@
 //
 // Same contract as ginn/dev.h:55-75: a Device allocates, frees and copies
 // memory, has a kind (CPU / GPU / NULL_DEV), an id and a precedence used by
-// best_dev().  GpuDevice owns one context of libginn_hip.so (device index,
+// best_dev().  A GPU index has one context of libginn_hip.so (device index,
 // stream, workspace) in place of the reference's stream + BLAS handle pair
-// (ginn/dev.h:149-199); PreallocGpuDevice is a bump arena in device memory
+// (ginn/dev.h:149-199), shared by all device objects of that index; PreallocGpuDevice is a bump arena in device memory
 // (ginn/dev.h:214-254).  Only the GPU kinds compute; CpuDevice holds host
 // staging copies of tensors.
 #ifndef GINN_DEV_H
@@ -110,20 +110,42 @@ class PreallocCpuDevice : public Device {
 
 inline auto PreallocCpu(size_t size) { return std::make_shared<PreallocCpuDevice>(size); }
 
-// One physical GPU: a libginn_hip.so context with its own stream.
-class GpuDevice : public Device {
-  const size_t id_;
-  ginn_hip_ctx* ctx_ = nullptr;
+namespace internal {
+// One context (stream, workspace) per GPU index for the whole process: every
+// device object of that index -- gpu(idx), a Gpu(idx) the caller made, a
+// PreallocGpu arena -- enqueues on it, so synchronising any of them waits for
+// the work on that GPU's tensors.  Created on first use and kept until the
+// process ends: tensors in static storage may free their memory later than
+// any static destructor of this header would run.
+class ContextTable {
+  std::vector<ginn_hip_ctx*> ctx_;
 
  public:
-  explicit GpuDevice(size_t id = 0) : id_(id) {
-    GINN_HIP_CALL(ginn_hip_ctx_create(static_cast<int>(id), 0, &ctx_));
+  ContextTable() : ctx_(static_cast<size_t>(std::max(gpus(), 0)), nullptr) {}
+  ContextTable(const ContextTable&) = delete;
+  ginn_hip_ctx*& at(size_t idx) {
+    GINN_ASSERT(idx < ctx_.size(),
+                "no GPU with index " + std::to_string(idx) + " (" + std::to_string(ctx_.size()) + " visible)");
+    if (!ctx_[idx]) GINN_HIP_CALL(ginn_hip_ctx_create(static_cast<int>(idx), 0, &ctx_[idx]));
+    return ctx_[idx];
   }
+};
+inline ContextTable& contexts() {
+  static ContextTable* table = new ContextTable;
+  return *table;
+}
+}  // namespace internal
+
+// One physical GPU.  Allocations are plain device allocations; kernels, copies
+// and synchronisation go to the GPU's process-wide context.
+class GpuDevice : public Device {
+  const size_t id_;
+  ginn_hip_ctx*& ctx_;
+
+ public:
+  explicit GpuDevice(size_t id = 0) : id_(id), ctx_(internal::contexts().at(id)) {}
   GpuDevice(const GpuDevice&) = delete;
   GpuDevice& operator=(const GpuDevice&) = delete;
-  ~GpuDevice() override {
-    if (ctx_) ginn_hip_ctx_destroy(ctx_);  // teardown never throws (ginn/dev.h:194-198)
-  }
 
   void* alloc(size_t size) override {
     void* p = nullptr;
@@ -167,8 +189,8 @@ inline auto& gpu(int idx = 0) {
 
 // The context that runs kernels for device index idx (role of cublas_handle(idx),
 // ginn/dev.h:264).
-inline ginn_hip_ctx* hip_ctx(int idx = 0) { return gpu(idx)->ctx(); }
-inline ginn_hip_ctx*& cublas_handle(int idx = 0) { return gpu(idx)->handle(); }
+inline ginn_hip_ctx* hip_ctx(int idx = 0) { return internal::contexts().at(static_cast<size_t>(idx)); }
+inline ginn_hip_ctx*& cublas_handle(int idx = 0) { return internal::contexts().at(static_cast<size_t>(idx)); }
 
 // Bump arena in device memory; kernels run on the context of gpu(id).
 class PreallocGpuDevice : public Device {
@@ -176,8 +198,11 @@ class PreallocGpuDevice : public Device {
   ginn_hip_arena* arena_ = nullptr;
 
  public:
-  PreallocGpuDevice(size_t id, size_t size) : id_(id) {
+  // alignment = 1 is the reference's byte-exact bump (ginn/dev.h:236-248);
+  // a larger power of two starts every block at a multiple of it.
+  PreallocGpuDevice(size_t id, size_t size, size_t alignment = 1) : id_(id) {
     GINN_HIP_CALL(ginn_hip_arena_create(hip_ctx(static_cast<int>(id)), size, &arena_));
+    if (alignment != 1) GINN_HIP_CALL(ginn_hip_arena_set_alignment(arena_, alignment));
   }
   explicit PreallocGpuDevice(size_t size) : PreallocGpuDevice(0, size) {}
   PreallocGpuDevice(const PreallocGpuDevice&) = delete;
@@ -209,6 +234,10 @@ class PreallocGpuDevice : public Device {
 
 inline auto PreallocGpu(size_t id, size_t size) { return std::make_shared<PreallocGpuDevice>(id, size); }
 inline auto PreallocGpu(size_t size) { return std::make_shared<PreallocGpuDevice>(size); }
+// Not in the reference: an arena whose blocks start at multiples of `alignment` bytes.
+inline auto PreallocGpuAligned(size_t id, size_t size, size_t alignment) {
+  return std::make_shared<PreallocGpuDevice>(id, size, alignment);
+}
 
 // Host <-> device and device <-> device transfers (ginn/dev.h:269-343).  One
 // GPU per process in this build: a copy between two different GPU indices is

@@ -235,6 +235,9 @@ class LevelExecutor {
       plan.capacity = bytes;
     }
     GINN_HIP_CALL(ginn_hip_memcpy_h2d(ctx_, plan.dev, blob.data(), bytes));
+    // The blob is reused by the next rebuild and the copy is only ordered on the
+    // stream: wait for it (plans are rebuilt when a graph changes, not per pass).
+    GINN_HIP_CALL(ginn_hip_sync(ctx_));
   }
 
   void launch(const Plan& plan) { launch(plan, 0, plan.launches.size()); }

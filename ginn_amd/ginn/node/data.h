@@ -90,6 +90,22 @@ class DataNode : public BaseDataNode<Scalar> {
 template <typename Scalar = Real>
 using DataPtr = Ptr<DataNode<Scalar>>;
 
+// A constant with the shape its input has at forward time; no gradient flows
+// through it (ginn/node/data.h:119-137).
+template <typename Scalar = Real>
+class ConstantLikeNode : public BaseDataNode<Scalar> {
+  Scalar val_;
+
+  void forward_() override {
+    this->value().resize(this->in()->shape());
+    this->value().fill(val_);
+  }
+
+ public:
+  ConstantLikeNode(NodePtr<Scalar> in, Real val) : BaseDataNode<Scalar>({in}), val_(val) {}
+  std::string name() const override { return "ConstantLike"; }
+};
+
 GINN_MAKE_TEMPLATE_FACTORY(Data);
 
 template <typename Scalar = Real>
@@ -131,6 +147,41 @@ auto FixedRandom(DevPtr dev, const Shape& shape) {
   auto x = FixedData<Scalar>(dev, shape);
   x->value().set_random();
   return x;
+}
+
+template <typename Scalar, typename InScalar>
+auto ConstantLike(NodePtr<InScalar> x, Scalar val) {
+  return make_ptr<ConstantLikeNode<Scalar>>(x, val);
+}
+template <typename Scalar>
+auto ZeroLike(NodePtr<Scalar> x) {
+  return ConstantLike<Scalar>(x, Scalar(0));
+}
+template <typename Scalar>
+auto OnesLike(NodePtr<Scalar> x) {
+  return ConstantLike<Scalar>(x, Scalar(1));
+}
+// The derived-pointer forms that callers have in hand (Ptr<DataNode<S>> etc.).
+template <typename NodeType, typename Scalar = typename NodeType::Scalar>
+auto ZeroLike(const Ptr<NodeType>& x) {
+  return ZeroLike<Scalar>(NodePtr<Scalar>(x));
+}
+template <typename NodeType, typename Scalar = typename NodeType::Scalar>
+auto OnesLike(const Ptr<NodeType>& x) {
+  return OnesLike<Scalar>(NodePtr<Scalar>(x));
+}
+
+// Values<2>({{1, 2, 3}, {4, 5, 6}}): a 2 x 3 data node from a literal, outermost
+// list = dimension 0 (ginn/node/data.h:211-221).
+template <int Rank, typename Scalar = Real>
+auto Values(DevPtr dev, NestedInitList<Rank, Scalar> val) {
+  auto x = Data<Scalar>(std::move(dev), shape_of<Size, Rank, Scalar>(val));
+  x->value().template set<Rank>(val);
+  return x;
+}
+template <int Rank, typename Scalar = Real>
+auto Values(NestedInitList<Rank, Scalar> val) {
+  return Values<Rank, Scalar>(cpu(), val);
 }
 
 // Data node with the given shape and values in storage (column-major) order.

@@ -71,6 +71,35 @@ GINN_MAKE_UNARY_NODE_AND_FACTORY(Sqrt);
 GINN_MAKE_UNARY_NODE_AND_FACTORY(Gelu);
 GINN_MAKE_UNARY_NODE_AND_FACTORY(Gelu2);
 
+// The same node writing over its input: value() and grad() are the input's
+// tensors, the backward pass rescales the gradient where it is instead of
+// adding to it (ginn/node/nlnode.h:72-97).
+#define GINN_MAKE_INPLACE_UNARY_NODE_AND_FACTORY(F)                            \
+  template <typename Scalar>                                                   \
+  class InPlace##F##Node : public F##Node<Scalar> {                            \
+   protected:                                                                  \
+    using F##Node<Scalar>::in_;                                                \
+    using F##Node<Scalar>::op_;                                                \
+    void backward_() override {                                                \
+      if (in_->has_grad()) op_.backward(in_->grad(), in_->grad(), in_->value(), in_->value(), false); \
+    }                                                                          \
+                                                                               \
+   public:                                                                     \
+    const Tensor<Scalar>& value() const override { return std::as_const(*in_).value(); } \
+    const Tensor<Scalar>& grad() const override { return std::as_const(*in_).grad(); }   \
+    using Node<Scalar>::value;                                                 \
+    using Node<Scalar>::grad;                                                  \
+    bool has_grad() const override { return in_->has_grad(); }                 \
+    bool describe_forward(std::vector<LaunchDesc>&) override { return false; } \
+    bool describe_backward(std::vector<LaunchDesc>&) override { return false; } \
+    using UnaryOp = F##Op<Scalar>;                                             \
+    using F##Node<Scalar>::F##Node;                                            \
+    std::string name() const override { return "InPlace" #F; }                 \
+  };                                                                           \
+  GINN_MAKE_SCALAR_FORWARDING_FACTORY(InPlace##F)
+
+GINN_MAKE_INPLACE_UNARY_NODE_AND_FACTORY(Sigmoid);
+
 }  // namespace ginn
 
 #endif  // GINN_NODE_NLNODE_H

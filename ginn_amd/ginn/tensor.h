@@ -16,6 +16,7 @@
 #include <utility>
 
 #include <ginn/dev.h>
+#include <ginn/util/util.h>
 
 namespace ginn {
 
@@ -102,6 +103,17 @@ class Tensor {
   }
   Tensor(DevPtr dev, Shape shape, const std::vector<Scalar>& val) : Tensor(std::move(shape), val) {
     move_to(dev);
+  }
+
+  // Tensor literals: Tensor<Real>(NestedInitList<2, Real>{{1, 2, 3}, {4, 5, 6}}) is 2 x 3
+  // (ginn/tensor.h:178-188).
+  template <int Rank>
+  Tensor(DevPtr dev, NestedInitList<Rank, Scalar> val) : dev_(std::move(dev)) {
+    set<Rank>(val);
+  }
+  template <int Rank>
+  Tensor(NestedInitList<Rank, Scalar> val) : dev_(cpu()) {
+    set<Rank>(val);
   }
 
   Tensor(const Tensor& other) : dev_(other.dev_), shape_(other.shape_) {
@@ -301,6 +313,40 @@ class Tensor {
     GINN_ASSERT(static_cast<Size>(vals.size()) == size());
     if (size() > 0)
       dev_->copy(*cpu(), data_, const_cast<Scalar*>(vals.data()), vals.size() * sizeof(Scalar));
+  }
+
+  // The first min(size(), vals.size()) elements, converted (ginn/tensor.h:472-489).
+  template <typename RhsScalar, typename = std::enable_if_t<!std::is_same_v<RhsScalar, Scalar>>>
+  void set(const std::vector<RhsScalar>& vals) {
+    std::vector<Scalar> all = vector();
+    for (size_t i = 0; i < std::min(all.size(), vals.size()); ++i) all[i] = convert<Scalar>(vals[i]);
+    set(all);
+  }
+  // set(1, 2, 3): values in storage order (ginn/tensor.h:491-494).
+  template <typename First, typename... Rest,
+            typename = std::enable_if_t<std::is_arithmetic_v<First> || std::is_same_v<First, Scalar>>>
+  void set(const First& first, const Rest&... rest) {
+    std::vector<Scalar> all = vector();
+    const std::vector<Scalar> vals{convert<Scalar>(first), convert<Scalar>(rest)...};
+    for (size_t i = 0; i < std::min(all.size(), vals.size()); ++i) all[i] = vals[i];
+    set(all);
+  }
+  // Resizes to the extents of the nested list and takes its values; element
+  // (i, j, ...) is val[i][j]... (ginn/tensor.h:496-510).
+  template <int Rank, typename RhsScalar = Scalar>
+  void set(NestedInitList<Rank, RhsScalar> val) {
+    const Shape shape = shape_of<Size, Rank, RhsScalar>(val);
+    resize(shape);
+    std::vector<Scalar> host(static_cast<size_t>(size()));
+    if (size() > 0) store_nested<Rank, Scalar, RhsScalar, Size>(val, host.data(), shape);
+    set(host);
+  }
+
+  template <typename To, typename From>
+  static To convert(const From& x) {
+    if constexpr (is_floating_point_v<To> && !std::is_same_v<To, float>) return To(static_cast<float>(x));
+    else if constexpr (is_floating_point_v<From>) return static_cast<To>(static_cast<float>(x));
+    else return static_cast<To>(x);
   }
 
   // this += other, elementwise, same device.

@@ -126,13 +126,22 @@ int ginn_hip_memset(ginn_hip_ctx* ctx, void* dst, int byte_value, size_t bytes);
 
 /* PreallocGpuDevice (ginn/dev.h:214-254): one slab, bump allocation, no
  * per-allocation free, clear() rewinds.  As in the reference an allocation
- * must leave at least one byte unused (`<`, not `<=`, ginn/dev.h:238-241).
- * Returned pointers are 256-byte aligned. */
+ * must leave at least one byte unused (`<`, not `<=`, ginn/dev.h:238-241),
+ * and as there the bump is byte-exact: used() is the sum of the sizes asked
+ * for, and a block starts where the last one ended (the slab itself is
+ * 256-byte aligned).  Every kernel of this library takes operands at any
+ * element-aligned address and falls back from 16-byte to element accesses
+ * when a pointer is not 16-byte aligned. */
 int ginn_hip_arena_create(ginn_hip_ctx* ctx, size_t bytes,
                           ginn_hip_arena** arena);
 int ginn_hip_arena_destroy(ginn_hip_arena* arena);
 int ginn_hip_arena_alloc(ginn_hip_arena* arena, size_t bytes, void** ptr);
 int ginn_hip_arena_clear(ginn_hip_arena* arena);
+/* No counterpart in the reference: from now on every block starts at a
+ * multiple of `alignment` bytes (a power of two <= 4096; 1 restores the
+ * byte-exact bump), so that tensors of mixed scalar types stay aligned and
+ * the 16-byte access paths are taken; the padding counts as used. */
+int ginn_hip_arena_set_alignment(ginn_hip_arena* arena, size_t alignment);
 int ginn_hip_arena_used(const ginn_hip_arena* arena, size_t* bytes);
 int ginn_hip_arena_size(const ginn_hip_arena* arena, size_t* bytes);
 

@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include <ginn/ginn.h>
@@ -274,6 +275,43 @@ int shim_executor_graph(int rows, int cols, int hidden, int replays, const float
     g_error = e.what();
     return 1;
   }
+}
+
+// Two host threads drive the one context of gpu(0) at the same time
+// (ginn/dev.h:203-212 hands every thread the same device object;
+// examples/bench.cu.cpp:442-445 and mnist-dp.cu:158-172 do exactly this).
+// Thread t computes C_t += A_t * B_t `iters` times through gpu_prod; the
+// shapes are chosen by the caller so that the products keep partial sums in
+// the context's workspace (split-K), which both threads share.  Outputs: C_0
+// and C_1 after the last iteration (expected: iters * A_t * B_t).
+int shim_two_threads(int dtype, int iters, const long* mnk0, const float* a0, const float* b0, float* c0,
+                     const long* mnk1, const float* a1, const float* b1, float* c1) {
+  DISPATCH(dtype, ([&]() -> int {
+    const long* mnk[2] = {mnk0, mnk1};
+    const float* as[2] = {a0, a1};
+    const float* bs[2] = {b0, b1};
+    float* cs[2] = {c0, c1};
+    std::string errors[2];
+    auto work = [&](int t) {
+      try {
+        auto A = make_data<S>({mnk[t][0], mnk[t][2]}, as[t], false);
+        auto B = make_data<S>({mnk[t][2], mnk[t][1]}, bs[t], false);
+        Tensor<S> C(gpu(), {mnk[t][0], mnk[t][1]});
+        C.set_zero();
+        for (int i = 0; i < iters; ++i)
+          internal::gpu_prod(C, A->value(), B->value(), internal::ProdResult::Add);
+        gpu()->synchronize();
+        read_back(C, cs[t]);
+      } catch (const std::exception& e) {
+        errors[t] = e.what();
+      }
+    };
+    std::thread other(work, 1);
+    work(0);
+    other.join();
+    if (!errors[0].empty() || !errors[1].empty()) throw std::runtime_error(errors[0] + " " + errors[1]);
+    return 0;
+  })());
 }
 
 // Error paths of the host layer that need no kernel: returns the message of

@@ -1,0 +1,406 @@
+// Structural checks of the host layer, run on the HIP device: what the
+// reference pins in test/tensor.cu.cpp (construction, copy, move, assignment
+// across devices, resize, set, serialize, errors), test/graph.cpp:26-115
+// (forwardedness, gradfulness, init_grad rules) and test/dev.cu.cpp:122-178
+// (byte accounting of the preallocated device arena, tensors and nodes).
+// The checks are written against the same public API a program written for the
+// reference uses (Values<2>({{..}}), Tensor(dev, {shape}, {values}), x + y,
+// Graph, PreallocGpu).  A failed check is recorded with its line and text;
+// pytest calls shim_structural(case) and expects an empty report.
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include <ginn/ginn.h>
+
+using namespace ginn;
+using namespace ginn::literals;
+
+namespace {
+
+thread_local std::string g_report;
+
+#define CHECK(cond)                                                             \
+  do {                                                                          \
+    if (!(cond)) g_report += std::string("line ") + std::to_string(__LINE__) + ": " #cond "\n"; \
+  } while (0)
+#define CHECK_THROWS(stmt)                                                      \
+  do {                                                                          \
+    bool thrown__ = false;                                                      \
+    try {                                                                       \
+      stmt;                                                                     \
+    } catch (const ginn::RuntimeError&) {                                       \
+      thrown__ = true;                                                          \
+    }                                                                           \
+    if (!thrown__) g_report += std::string("line ") + std::to_string(__LINE__) + ": no RuntimeError from " #stmt "\n"; \
+  } while (0)
+
+template <typename Scalar>
+std::vector<Scalar> one_to_six() {
+  std::vector<Scalar> v;
+  for (int i = 1; i <= 6; ++i) v.push_back(Scalar(i));
+  return v;
+}
+
+template <typename Scalar>
+Scalar sample_value() {
+  if constexpr (std::is_same_v<Scalar, Int>) return 4;
+  else return Scalar(0.6f);
+}
+
+template <typename Scalar>
+bool all_equal(const Tensor<Scalar>& t, float val) {
+  for (const Scalar& x : t.vector())
+    if (!(static_cast<float>(x) == val)) return false;
+  return true;
+}
+
+enum Maker { PLAIN, COPIED, MOVED, ASSIGNED_TO_GPU, ASSIGNED_TO_CPU };
+
+// The five ways of obtaining a tensor from the same constructor arguments
+// (test/tensor.cu.cpp:33-49), each checked for device, size, rank and values.
+template <typename Scalar, typename... Args>
+void made(Maker how, DeviceKind expect, Size size, size_t rank, const float* val, DevPtr init, Args... args) {
+  using T = Tensor<Scalar>;
+  auto check = [&](T& t) {
+    CHECK(t.dev()->kind() == expect);
+    CHECK(t.size() == size);
+    if (rank) CHECK(t.shape().size() == rank);
+    if (val) {
+      t.move_to(cpu());
+      for (Size i = 0; i < t.size(); ++i) CHECK(static_cast<float>(t.v()[i]) == *val);
+    }
+  };
+  if (how == PLAIN) {
+    T t(init, args...);
+    check(t);
+  } else if (how == COPIED) {
+    T t_(init, args...);
+    T t(t_);
+    check(t);
+  } else if (how == MOVED) {
+    T t_(init, args...);
+    T t(std::move(t_));
+    check(t);
+  } else {
+    T t_(init, args...);
+    T t(how == ASSIGNED_TO_GPU ? DevPtr(gpu()) : DevPtr(cpu()));
+    t = t_;
+    check(t);
+  }
+}
+
+template <typename Scalar>
+void tensor_ctors() {
+  struct Row { Maker how; bool init_gpu; DeviceKind expect; };
+  const Row rows[] = {{PLAIN, false, CPU}, {COPIED, false, CPU}, {MOVED, false, CPU}, {ASSIGNED_TO_CPU, false, CPU},
+                      {PLAIN, true, GPU},  {COPIED, true, GPU},  {MOVED, true, GPU},  {ASSIGNED_TO_GPU, true, GPU},
+                      {ASSIGNED_TO_CPU, true, CPU}};
+  const Scalar val = sample_value<Scalar>();
+  const float fval = static_cast<float>(val);
+  for (const Row& r : rows) {
+    const DevPtr init = r.init_gpu ? DevPtr(gpu()) : DevPtr(cpu());
+    made<Scalar>(r.how, r.expect, 0, 0, nullptr, init);
+    made<Scalar>(r.how, r.expect, 6, 3, nullptr, init, Shape{2, 1, 3});
+    made<Scalar>(r.how, r.expect, 6, 3, &fval, init, Shape{2, 1, 3}, val);
+  }
+}
+
+template <typename Scalar, typename DeviceType>
+void tensor_resize_set_serialize_errors() {
+  using T = Tensor<Scalar>;
+  auto dev = std::make_shared<DeviceType>();
+  auto fresh = [&] {
+    T t(dev);
+    t = T(dev, {2, 1, 3}, one_to_six<Scalar>());
+    return t;
+  };
+  auto counts_up = [&](T& t) {
+    t.move_to(cpu());
+    for (Size i = 0; i < t.size(); ++i) CHECK(static_cast<float>(t.v()[i]) == static_cast<float>(i + 1));
+  };
+  {  // same size: contents stay
+    T t = fresh();
+    t.resize({6});
+    CHECK(t.size() == 6);
+    CHECK((t.shape() == Shape{6}));
+    counts_up(t);
+  }
+  {
+    T t = fresh();
+    t.resize({2, 3});
+    CHECK((t.shape() == Shape{2, 3}));
+    counts_up(t);
+  }
+  {
+    T t = fresh();
+    t.resize({4});
+    CHECK(t.size() == 4);
+    CHECK((t.shape() == Shape{4}));
+    t.resize({2, 2});
+    CHECK((t.shape() == Shape{2, 2}));
+  }
+  {  // host access only on host tensors
+    T t = fresh();
+    if (dev->kind() == CPU) {
+      CHECK(t.v() == t.data());
+    } else {
+      CHECK_THROWS(t.v());
+    }
+    // folds of the shape (views of rank 1..5 in the reference)
+    CHECK((T::reduce(t.shape(), 1) == Shape{6}));
+    CHECK((T::reduce(t.shape(), 2) == Shape{2, 3}));
+    CHECK((T::reduce(t.shape(), 3) == Shape{2, 1, 3}));
+    CHECK((T::reduce(t.shape(), 5) == Shape{2, 1, 3, 1, 1}));
+    CHECK(t.rows() == 2 && t.cols() == 3);
+  }
+  {
+    T t = fresh();
+    t.set_zero();
+    CHECK(all_equal(t, 0.f));
+    t.set_ones();
+    CHECK(all_equal(t, 1.f));
+    Scalar val;
+    if constexpr (std::is_same_v<Scalar, Int>) val = 12345;
+    else val = Scalar(0.12345f);
+    t.fill(val);
+    CHECK(all_equal(t, static_cast<float>(val)));
+  }
+  if constexpr (std::is_same_v<Scalar, Real>) {
+    T t = fresh();
+    t.set_random();
+    t.move_to(cpu());
+    for (Size i = 0; i < t.size(); ++i) {
+      CHECK(t.v()[i] <= 1.f && t.v()[i] >= -1.f);
+      if (i > 0) CHECK(t.v()[i] != t.v()[i - 1]);
+    }
+  }
+  {  // set(values...): as many as fit, the rest stays
+    T t = fresh();
+    t.set(5, 4, 3, 2, 1, 0);
+    auto v = t.vector();
+    for (size_t i = 0; i < v.size(); ++i) CHECK(static_cast<float>(v[i]) == 5.f - static_cast<float>(i));
+    t.set(5, 4, 3, 2, 1, 0, 1, 2, 3);
+    v = t.vector();
+    for (size_t i = 0; i < v.size(); ++i) CHECK(static_cast<float>(v[i]) == 5.f - static_cast<float>(i));
+    T u = fresh();
+    u.set(5, 4, 3);
+    v = u.vector();
+    const float want[6] = {5, 4, 3, 4, 5, 6};
+    for (size_t i = 0; i < 6; ++i) CHECK(static_cast<float>(v[i]) == want[i]);
+  }
+  {  // nested literal: element (i, j) is list[i][j]
+    T t(dev);
+    t.template set<2>(NestedInitList<2, Scalar>{{Scalar(1), Scalar(2), Scalar(3)}, {Scalar(4), Scalar(5), Scalar(6)}});
+    CHECK((t.shape() == Shape{2, 3}));
+    const auto v = t.vector();
+    const float want[6] = {1, 4, 2, 5, 3, 6};  // column-major storage
+    for (size_t i = 0; i < 6; ++i) CHECK(static_cast<float>(v[i]) == want[i]);
+  }
+  {
+    T t = fresh(), t2(dev);
+    std::ostringstream out;
+    t.save(out);
+    std::istringstream in(out.str());
+    t2.load(in);
+    CHECK(t == t2);
+  }
+  {
+    T t1(dev, {1, 2}), t2(dev, {1, 3}), t3(dev);
+    t3.map(t1, {2, 1});
+    CHECK_THROWS(t3 = t2);
+    CHECK_THROWS(t3.map(t2, {2, 1}));
+    std::string msg;
+    try {
+      T bad(Shape{1, 3}, std::vector<Scalar>{Scalar(1), Scalar(2)});
+    } catch (const ginn::RuntimeError& e) {
+      msg = e.what();
+    }
+    CHECK(msg == "Size of Shape (3) does not match size of values (2)!");
+  }
+}
+
+// test/graph.cpp:26-54, on the device (nodes compute there in this build).
+void forwardedness() {
+  auto make = [] {
+    auto a = Identity(Data(gpu(), {2, 3}));
+    auto b = Identity(Data(gpu(), {2, 3}));
+    return std::make_pair(a, b);
+  };
+  {
+    auto [a, b] = make();
+    auto c = a + b;
+    Graph g(c);
+    CHECK(g.nodes().size() == 5);
+    g.forward();
+    for (const auto& e : g.nodes()) CHECK(e->forwarded);
+  }
+  {
+    auto [a, b] = make();
+    auto c = a + b;
+    Graph(a).forward();
+    CHECK(a->forwarded);
+    CHECK(!b->forwarded);
+    CHECK(!c->forwarded);
+  }
+  {
+    auto [a, b] = make();
+    auto c = a + b;
+    Graph g(c);
+    auto d = c + a;
+    g.forward();
+    for (const auto& e : g.nodes()) CHECK(e->forwarded);
+    CHECK(!d->forwarded);
+  }
+}
+
+// test/graph.cpp:56-113.
+void gradfulness() {
+  auto a = Random(gpu(), {2, 3});
+  auto b = FixedRandom(gpu(), {2, 3});
+  auto c = a + b;
+  Graph g(c);
+  CHECK(a->has_grad());
+  CHECK(!b->has_grad());
+  CHECK(c->has_grad());
+  CHECK(a->grad().size() == 0);
+  CHECK(b->grad().size() == 0);
+  CHECK(c->grad().size() == 0);
+
+  g.forward();
+  g.init_grad();
+  CHECK((a->grad().shape() == Shape{2, 3}));
+  CHECK(b->grad().size() == 0);
+  CHECK((c->grad().shape() == Shape{2, 3}));
+
+  a->grad().fill(3.f);
+  g.reset_grad();
+  CHECK((a->grad().shape() == Shape{2, 3}));
+  CHECK(all_equal(a->grad(), 0.f));
+  CHECK(b->grad().size() == 0);
+  CHECK(all_equal(c->grad(), 0.f));
+
+  // init_grad keeps a gradient of the right size ...
+  a->grad() = Tensor<Real>(gpu(), {2, 3}, {1, 2, 3, 4, 5, 6});
+  g.init_grad();
+  const auto kept = a->grad().vector();
+  for (size_t i = 0; i < 6; ++i) CHECK(kept[i] == static_cast<float>(i + 1));
+  // ... and replaces one of the wrong size
+  a->grad() = Tensor<Real>(gpu(), {1, 3}, {1, 2, 3});
+  g.init_grad();
+  CHECK((a->grad().shape() == Shape{2, 3}));
+}
+
+// test/dev.cu.cpp:122-155: the arena counts exactly the bytes asked for.
+template <typename Scalar>
+void arena_tensors() {
+  auto dev = PreallocGpu(100);
+  Tensor<Scalar> t1(gpu(), {2, 3});
+  CHECK(dev->used() == 0);
+  Tensor<Scalar> t2(dev, {1, 2});
+  CHECK(dev->used() == t2.size() * sizeof(Scalar));
+  Tensor<Scalar> t3(dev);
+  CHECK(dev->used() == t2.size() * sizeof(Scalar));
+  t3 = t2;  // copies
+  CHECK(dev->used() == 2 * t2.size() * sizeof(Scalar));
+  auto t4 = t1.maybe_copy_to(dev);  // same GPU: a view, no copy
+  CHECK(dev->used() == 2 * t2.size() * sizeof(Scalar));
+  t1.move_to(dev);
+  CHECK(dev->used() == (2 * t2.size() + t1.size()) * sizeof(Scalar));
+  t2.move_to(dev);  // already there
+  CHECK(dev->used() == (2 * t2.size() + t1.size()) * sizeof(Scalar));
+  Tensor<Scalar> t5(cpu(), {1, 3});
+  auto t6 = t5.maybe_copy_to(dev);  // from the host: a copy
+  CHECK(dev->used() == (2 * t2.size() + t1.size() + t5.size()) * sizeof(Scalar));
+  CHECK(dev->size() == 100);
+  dev->clear();
+  CHECK(dev->used() == 0);
+}
+
+// test/dev.cu.cpp:157-178, with the result of x + y checked as well: the
+// operands sit back to back in the arena, 24 or 12 bytes apart.
+template <typename Scalar>
+void arena_nodes() {
+  auto dev = PreallocGpu(200);
+  auto x = Values<2>({{1, 2, 3}, {4, 5, 6}})->cast<Scalar>();
+  auto y = Values<2>({{1, 2, 3}, {4, 5, 6}})->cast<Scalar>();
+  x->set_has_grad(false);
+  CHECK(dev->used() == 0);
+  x->move_to(dev);
+  CHECK(dev->used() == x->size() * sizeof(Scalar));
+  y->move_to(dev);  // value and (empty) gradient
+  CHECK(dev->used() == 2 * x->size() * sizeof(Scalar));
+  auto z = x + y;
+  Graph g(z);
+  CHECK(dev->used() == 2 * x->size() * sizeof(Scalar));
+  g.forward();
+  CHECK(dev->used() == 3 * x->size() * sizeof(Scalar));
+  g.reset_grad();  // z and y have gradients, x does not
+  CHECK(dev->used() == 5 * x->size() * sizeof(Scalar));
+  const auto v = z->value().vector();
+  const float want[6] = {2, 8, 4, 10, 6, 12};
+  for (size_t i = 0; i < 6; ++i) CHECK(static_cast<float>(v[i]) == want[i]);
+  g.backward(1.);
+  CHECK(all_equal(y->grad(), 1.f));
+}
+
+// A block that does not fit leaves the arena as it was; aligned arenas pad.
+void arena_limits() {
+  auto dev = PreallocGpu(100);
+  Tensor<Real> a(dev, {24});  // 96 bytes: fits (96 < 100)
+  CHECK(dev->used() == 96);
+  CHECK_THROWS(Tensor<Real>(dev, {1}));  // 96 + 4 is not < 100
+  CHECK(dev->used() == 96);
+  auto al = PreallocGpuAligned(0, 1024, 256);
+  Tensor<Half> h(al, {3});
+  Tensor<Real> r(al, {2});
+  CHECK(al->used() == 256 + 8);
+  CHECK(reinterpret_cast<uintptr_t>(r.data()) % 256 == 0);
+}
+
+}  // namespace
+
+extern "C" {
+
+// Runs the named group of checks; returns the report of failed checks ("" = all passed).
+const char* shim_structural(const char* which) {
+  g_report.clear();
+  const std::string w(which);
+  try {
+    if (w == "tensor_ctors") {
+      tensor_ctors<Real>();
+      tensor_ctors<Int>();
+      tensor_ctors<Half>();
+      tensor_ctors<BFloat16>();
+    } else if (w == "tensor_ops") {
+      tensor_resize_set_serialize_errors<Real, GpuDevice>();
+      tensor_resize_set_serialize_errors<Int, GpuDevice>();
+      tensor_resize_set_serialize_errors<Half, GpuDevice>();
+      tensor_resize_set_serialize_errors<BFloat16, GpuDevice>();
+      tensor_resize_set_serialize_errors<Real, CpuDevice>();
+      tensor_resize_set_serialize_errors<Int, CpuDevice>();
+      tensor_resize_set_serialize_errors<Half, CpuDevice>();
+    } else if (w == "forwardedness") {
+      forwardedness();
+    } else if (w == "gradfulness") {
+      gradfulness();
+    } else if (w == "arena_tensors") {
+      arena_tensors<Real>();
+      arena_tensors<Int>();
+      arena_tensors<Half>();
+    } else if (w == "arena_nodes") {
+      arena_nodes<Real>();
+      arena_nodes<Half>();
+      arena_nodes<BFloat16>();
+    } else if (w == "arena_limits") {
+      arena_limits();
+    } else {
+      g_report = "unknown case " + w;
+    }
+  } catch (const std::exception& e) {
+    g_report += std::string("exception: ") + e.what() + "\n";
+  }
+  return g_report.c_str();
+}
+
+}  // extern "C"

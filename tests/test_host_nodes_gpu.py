@@ -71,6 +71,45 @@ def test_prod_nodes(shim, dt, a_shape, b_shape, batched):
     assert rel_fro(db, 2 * want_db) <= TOL[dt] * 2
 
 
+@pytest.mark.parametrize("dt", [capi.F16, capi.BF16])
+@pytest.mark.parametrize("product", ["QK^T", "PV"])
+def test_attention_products_through_batched_prod_node(shim, dt, product):
+    """The attention configuration at its stated size: batch * heads = 128 slices,
+    QK^T = [256 x 64] * [64 x 256] and P V = [256 x 256] * [256 x 64] with Q, K,
+    V ~ N(0, 1) and P the row-softmax of a seeded N(0, 1) matrix, 16-bit storage,
+    through BatchedProdNode (ginn/node/prod.h:93-169): value and both input
+    gradients (dA = dY B^T per slice, dB = A^T dY per slice) against the fp64
+    oracle, protocol of test/nodes.cu.cpp:1043-1115 (e = f() + f(), masked sum)."""
+    from gpu_util import TOL, round_to
+    rng = np.random.default_rng(4 if product == "PV" else 44)
+    batch = 128
+    if product == "QK^T":
+        a_shape, b_shape = (256, 64, batch), (64, 256, batch)
+        a = rng.standard_normal(a_shape)
+        b = rng.standard_normal(b_shape)
+    else:
+        a_shape, b_shape = (256, 256, batch), (256, 64, batch)
+        s = rng.standard_normal(a_shape)
+        e = np.exp(s - s.max(axis=1, keepdims=True))
+        a = e / e.sum(axis=1, keepdims=True)  # every row of every slice sums to 1
+        b = rng.standard_normal(b_shape)
+    a, b = round_to(a, dt), round_to(b, dt)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    want_f = N.batched_prod_forward(a64, b64)
+    mask = round_to(rng.uniform(-1, 1, want_f.shape), dt)
+    out = np.zeros(want_f.shape, np.float32, order="F")
+    da = np.zeros(a_shape, np.float32, order="F")
+    db = np.zeros(b_shape, np.float32, order="F")
+    check(shim, shim.shim_prod_node(dt, 1, dims(a_shape), 3, dims(b_shape), 3, fptr(f32(a)), fptr(f32(b)),
+                                    fptr(f32(mask)), fptr(out), fptr(da), fptr(db)))
+    want_da, want_db = N.batched_prod_backward(a64, b64, mask.astype(np.float64))
+    assert rel_fro(out, 2 * want_f) <= TOL[dt]
+    assert rel_fro(da, 2 * want_da) <= TOL[dt]
+    assert rel_fro(db, 2 * want_db) <= TOL[dt]
+    # independent of the oracle: slice 77 of the value is the plain product of slice 77
+    np.testing.assert_allclose(out[:, :, 77] / 2, a64[:, :, 77] @ b64[:, :, 77], rtol=0, atol=TOL[dt] * np.abs(want_f).max())
+
+
 @pytest.mark.parametrize("dt", DTYPES)
 def test_prod_reference_golden(shim, golden, dt):
     g = golden["prod"]
@@ -155,6 +194,46 @@ def test_nonlin_nodes(shim, dt, act):
     want_dx = N.nonlin_backward(act, mask.astype(np.float64), x.astype(np.float64), want)
     assert rel_fro(out, 2 * want) <= TOL[dt] * 2
     assert rel_fro(dx, 2 * want_dx) <= TOL[dt] * 4
+
+
+@pytest.mark.parametrize("case", ["tensor_ctors", "tensor_ops", "forwardedness", "gradfulness", "arena_tensors",
+                                  "arena_nodes", "arena_limits"])
+def test_reference_structural_cases(shim, case):
+    """The reference's structural tests on the HIP device: Tensor construction /
+    copy / move / assignment across devices, resize, set, serialize and errors
+    (test/tensor.cu.cpp), forwardedness and gradient allocation rules
+    (test/graph.cpp:26-115), and the byte accounting of the preallocated device
+    arena for tensors and nodes (test/dev.cu.cpp:122-178)."""
+    shim.shim_structural.restype = ctypes.c_char_p
+    report = shim.shim_structural(case.encode()).decode()
+    assert report == "", report
+
+
+@pytest.mark.parametrize("dt,shape0,shape1", [
+    (capi.F32, (512, 64, 784), (10, 64, 512)),       # generic kernel, split-K partials in the workspace
+    (capi.F32, (4096, 1, 4096), (4096, 16, 4096)),   # skinny kernels, K split over blocks
+    (capi.BF16, (768, 768, 4096), (4096, 1, 4096)),  # 128 x 128 family with split-K, and the 16-bit skinny kernel
+])
+def test_one_context_two_host_threads(shim, dt, shape0, shape1):
+    """Two host threads enqueue split-K products on the same context at the same
+    time; each keeps its partial sums in the context's one workspace.  Every
+    iteration accumulates into C, so one interleaved fold would show."""
+    from gpu_util import TOL, round_to
+    rng = np.random.default_rng(shape0[0] + shape1[1])
+    iters = 16
+    ops, outs = [], []
+    for m, n, k in (shape0, shape1):
+        a = round_to(rng.standard_normal((m, k)) / np.sqrt(k), dt)
+        b = round_to(rng.standard_normal((k, n)), dt)
+        ops.append((a, b))
+        outs.append(np.zeros((m, n), np.float32, order="F"))
+    args = []
+    for (a, b), (m, n, k), c in zip(ops, (shape0, shape1), outs):
+        args += [(ctypes.c_long * 3)(m, n, k), fptr(f32(a)), fptr(f32(b)), fptr(c)]
+    check(shim, shim.shim_two_threads(dt, iters, *args))
+    for (a, b), c in zip(ops, outs):
+        want = iters * (a.astype(np.float64) @ b.astype(np.float64))
+        assert rel_fro(c, want) <= TOL[dt]
 
 
 def test_error_paths(shim):
