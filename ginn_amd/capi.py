@@ -45,6 +45,8 @@ PROTOTYPES = {
     "ginn_hip_arena_size": (c_int, [c_void_p, POINTER(c_size_t)]),
     "ginn_hip_gemm": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                               c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_int]),
+    "ginn_hip_gemm_noalloc": (c_int, [c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                      c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_int]),
     "ginn_hip_gemm_strided_batched": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                               c_void_p, c_int, c_longlong, c_void_p, c_int, c_longlong,
                                               c_float, c_void_p, c_int, c_longlong, c_int]),

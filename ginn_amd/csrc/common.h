@@ -357,6 +357,10 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& args);
 // of `args` (beta, bias, activation, pre-activation) into C.
 int launch_splitk_reduce(ginn_hip_ctx* ctx, const GemmArgs& args, int splits, const float* partial);
 
+// Looks up, once per GPU and with that GPU current, the device address of the
+// scratch array behind ginn_hip_gemm_noalloc.
+void noalloc_prepare(int device);
+
 int launch_softmax_fwd(ginn_hip_ctx* ctx, int dtype, int rows, int cols,
                        const void* x, void* y);
 

@@ -55,6 +55,7 @@ int create_ctx(int device, hipStream_t stream, bool own_stream,
                "ginn_hip_ctx_create: device %d out of range (%d visible)",
                device, count);
   GH_HIP(hipSetDevice(device));
+  noalloc_prepare(device);
   ginn_hip_ctx* ctx = new (std::nothrow) ginn_hip_ctx();
   if (!ctx) return fail(kOutOfMemory, "ginn_hip_ctx_create: host allocation failed");
   ctx->device = device;

@@ -168,6 +168,30 @@ int ginn_hip_gemm_strided_batched(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
                                   long long stride_b, float beta, void* C,
                                   int ldc, long long stride_c, int batch);
 
+/* ginn_hip_gemm for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose BLAS handle allocates its workspace
+ * when it is created, ginn/dev.h:188-189).  Same product, same kernels; it
+ * takes a device index and a hipStream_t (NULL = the null stream) instead of
+ * a context, and the split-K partial sums live in a 16 MiB device array that
+ * is part of the library image (one copy per GPU, held until the process
+ * ends).  The call allocates and frees nothing: no hipMalloc, hipHostMalloc
+ * or hipFree, no context.
+ * Limit: m * n <= 2 097 152 output elements (two fp32 partial copies of the
+ * output fit the array) -- the small and skinny products of a serving loop;
+ * a larger output is refused with an error, use ginn_hip_gemm for it.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on
+ * one GPU (two streams, or two processes' worth of graphs replayed at once)
+ * race on it; calls on one stream, or on streams the caller orders, do not.
+ * The array's old contents never matter (partial sums are written before
+ * they are read).  The address of the array is looked up once per GPU, at
+ * the first ginn_hip_ctx_create on that GPU or at the first call of this
+ * function, whichever comes first: make that first use outside a capture. */
+int ginn_hip_gemm_noalloc(int device, void* stream, ginn_hip_dtype dtype,
+                          ginn_hip_op op_a, ginn_hip_op op_b, int m, int n,
+                          int k, const void* A, int lda, const void* B,
+                          int ldb, float beta, void* C, int ldc);
+
 /* One launch for `groups` products that share the left operand:
  * C_g[m x n_g] = op(A) * B_g[k x n_g] + beta * C_g.  This is the product
  * that Autobatch forms by concatenating right-hand sides
