@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import importlib.util
-from ctypes import (POINTER, byref, c_char_p, c_float, c_int, c_longlong,
+from ctypes import (POINTER, byref, c_char_p, c_float, c_int, c_longlong, c_ulonglong,
                     c_size_t, c_void_p)
 from pathlib import Path
 
@@ -84,6 +84,28 @@ PROTOTYPES = {
                                  c_int]),
     "ginn_hip_mask_fill": (c_int, [c_void_p, c_int, c_size_t, c_size_t, c_void_p, c_float, c_void_p]),
     "ginn_hip_upper_tri": (c_int, [c_void_p, c_int, c_int, c_void_p]),
+    "ginn_hip_layernorm_bwd_assign": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_elementwise": (c_int, [c_void_p, c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p, c_int]),
+    "ginn_hip_fill_uniform": (c_int, [c_void_p, c_int, c_size_t, c_ulonglong, c_float, c_float, c_void_p]),
+    "ginn_hip_dropout_mask": (c_int, [c_void_p, c_size_t, c_float, c_ulonglong, c_void_p]),
+    "ginn_hip_mask_scale": (c_int, [c_void_p, c_int, c_size_t, c_float, c_void_p, c_void_p, c_void_p, c_int]),
+    "ginn_hip_select": (c_int, [c_void_p, c_int, c_size_t, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
+    "ginn_hip_select_bwd": (c_int, [c_void_p, c_int, c_size_t, c_void_p, c_int, c_void_p, c_void_p, c_int]),
+    "ginn_hip_mask_select": (c_int, [c_void_p, c_int, c_size_t, c_size_t, c_void_p, c_float, c_void_p, c_void_p, c_int]),
+    "ginn_hip_less_than": (c_int, [c_void_p, c_int, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_pick": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_pick_bwd": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p]),
+    "ginn_hip_pick_nlsig_fwd": (c_int, [c_void_p, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_pick_nlsig_bwd": (c_int, [c_void_p, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_axis_sum": (c_int, [c_void_p, c_int, c_int, POINTER(c_longlong), POINTER(c_int), c_void_p, c_void_p]),
+    "ginn_hip_axis_sum_bwd": (c_int, [c_void_p, c_int, c_int, POINTER(c_longlong), POINTER(c_int), c_void_p, c_void_p]),
+    "ginn_hip_variance_fwd": (c_int, [c_void_p, c_int, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_variance_bwd": (c_int, [c_void_p, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_stack": (c_int, [c_void_p, c_int, c_size_t, c_size_t, c_void_p, c_void_p]),
+    "ginn_hip_stack_bwd": (c_int, [c_void_p, c_int, c_size_t, c_size_t, c_void_p, c_void_p]),
+    "ginn_hip_argmax": (c_int, [c_void_p, c_int, c_size_t, c_size_t, c_size_t, c_void_p, c_void_p]),
+    "ginn_hip_row_broadcast": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "ginn_hip_col_sum": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int]),
     "ginn_hip_multi_apply": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_float, c_size_t, c_int, c_void_p,
                                      c_void_p, c_void_p, c_void_p]),
     "ginn_hip_multi_mixed": (c_int, [c_void_p, c_int, c_void_p, c_size_t]),

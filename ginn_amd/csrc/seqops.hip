@@ -17,8 +17,8 @@ constexpr int kWaves = kBlock / 64;
 // as the reference evaluates them), then the normalised values.
 template <typename T, int V>
 __global__ __launch_bounds__(kBlock) void layernorm_fwd_kernel(int rows, int cols,
-                                                               const typename T::storage* __restrict__ x, float eps,
-                                                               typename T::storage* __restrict__ y,
+                                                               const typename T::storage* x, float eps,
+                                                               typename T::storage* y,  // may be x (in place)
                                                                float* __restrict__ std_out) {
   const int lane = threadIdx.x & 63;
   const int wave = blockIdx.x * kWaves + (threadIdx.x >> 6);
@@ -54,13 +54,16 @@ __global__ __launch_bounds__(kBlock) void layernorm_fwd_kernel(int rows, int col
   }
 }
 
-// dx += (dy - mean(dy) - y * (dy . y) / rows) / std, one wave per column.
+// dx (+)= (dy - mean(dy) - y * (dy . y) / rows) / std, one wave per column.
+// Without `accumulate`, dx may be dy itself (the in-place node): a lane reads
+// its elements of dy right before it writes the same elements of dx, after
+// the column's sums are complete.
 template <typename T, int V>
 __global__ __launch_bounds__(kBlock) void layernorm_bwd_kernel(int rows, int cols,
-                                                               const typename T::storage* __restrict__ dy,
+                                                               const typename T::storage* dy,
                                                                const typename T::storage* __restrict__ y,
                                                                const float* __restrict__ std_in,
-                                                               typename T::storage* dx) {
+                                                               typename T::storage* dx, int accumulate) {
   const int lane = threadIdx.x & 63;
   const int wave = blockIdx.x * kWaves + (threadIdx.x >> 6);
   const int nwaves = gridDim.x * kWaves;
@@ -85,7 +88,9 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_kernel(int rows, int col
       float g[V], yv[V], old[V];
       ld<T, V>(dy + base + r, g);
       ld<T, V>(y + base + r, yv);
-      ld<T, V>(dx + base + r, old);
+#pragma unroll
+      for (int e = 0; e < V; ++e) old[e] = 0.f;
+      if (accumulate) ld<T, V>(dx + base + r, old);
 #pragma unroll
       for (int e = 0; e < V; ++e) old[e] += (g[e] - gmean - yv[e] * dot) * inv;
       st<T, V>(dx + base + r, old);
@@ -409,20 +414,30 @@ int ginn_hip_layernorm_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, in
   return kOk;
 }
 
-int ginn_hip_layernorm_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* dy, const void* y,
-                           const float* std_in, void* dx) {
-  GH_CHECK_ARG(ctx, "ginn_hip_layernorm_bwd: ctx is NULL");
-  GH_CHECK_ARG(rows >= 0 && cols >= 0, "ginn_hip_layernorm_bwd: negative dimension");
+static int layernorm_bwd(const char* who, ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* dy,
+                         const void* y, const float* std_in, void* dx, int accumulate) {
+  GH_CHECK_ARG(ctx, "%s: ctx is NULL", who);
+  GH_CHECK_ARG(rows >= 0 && cols >= 0, "%s: negative dimension", who);
   if (rows == 0 || cols == 0) return kOk;
-  GH_CHECK_ARG(dy && y && std_in && dx, "ginn_hip_layernorm_bwd: NULL pointer");
+  GH_CHECK_ARG(dy && y && std_in && dx, "%s: NULL pointer", who);
   GH_HIP(hipSetDevice(ctx->device));
   const unsigned grid = grid_for(static_cast<size_t>(cols), kWaves, ctx->num_cus);
   const bool vec = vec8_ok({dy, y, dx}, {static_cast<size_t>(rows)});
   GH_DISPATCH_DTYPE_V(dtype, vec, (layernorm_bwd_kernel<T, V><<<grid, kBlock, 0, ctx->stream>>>(
       rows, cols, static_cast<const T::storage*>(dy), static_cast<const T::storage*>(y), std_in,
-      static_cast<T::storage*>(dx))));
+      static_cast<T::storage*>(dx), accumulate)));
   GH_HIP(hipGetLastError());
   return kOk;
+}
+
+int ginn_hip_layernorm_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* dy, const void* y,
+                           const float* std_in, void* dx) {
+  return layernorm_bwd("ginn_hip_layernorm_bwd", ctx, dtype, rows, cols, dy, y, std_in, dx, 1);
+}
+
+int ginn_hip_layernorm_bwd_assign(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* dy,
+                                  const void* y, const float* std_in, void* dx) {
+  return layernorm_bwd("ginn_hip_layernorm_bwd_assign", ctx, dtype, rows, cols, dy, y, std_in, dx, 0);
 }
 
 int ginn_hip_cwise_prod_add_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* a,

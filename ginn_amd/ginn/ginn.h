@@ -11,6 +11,7 @@
 #include <ginn/node.h>
 #include <ginn/node/affine.h>
 #include <ginn/node/common.h>
+#include <ginn/node/compare.h>
 #include <ginn/node/data.h>
 #include <ginn/node/inplace.h>
 #include <ginn/node/layernorm.h>
@@ -19,9 +20,12 @@
 #include <ginn/node/pick.h>
 #include <ginn/node/prod.h>
 #include <ginn/node/reduce.h>
+#include <ginn/node/select.h>
 #include <ginn/node/weight.h>
 #include <ginn/nonlin.h>
 #include <ginn/prod.h>
 #include <ginn/tensor.h>
+#include <ginn/util/amax.h>
+#include <ginn/util/util.h>
 
 #endif  // GINN_GINN_H

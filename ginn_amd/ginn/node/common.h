@@ -1,5 +1,6 @@
 // Arithmetic nodes used around the product path (ginn/node/common.h): N-ary
-// Add, CwiseProd, ProdScalar, AddScalar and the operator sugar for them.
+// Add, Subtract, CwiseProd, CwiseProdAdd, CwiseMax, ProdScalar, AddScalar,
+// SubtractScalar, Dropout and the operator sugar for them.
 #ifndef GINN_NODE_COMMON_H
 #define GINN_NODE_COMMON_H
 
@@ -100,6 +101,7 @@ GINN_MAKE_SCALAR_FORWARDING_FACTORY(Add);
 // value = a (*) b; backward da += dy (*) b, db += dy (*) a (ginn/node/common.h:233-262).
 template <typename Scalar>
 class CwiseProdNode : public BaseDataNode<Scalar> {
+ protected:
   NodePtr<Scalar> a_, b_;
 
   void run(Tensor<Scalar>& dst, const Tensor<Scalar>& x, const Tensor<Scalar>& y, bool acc) {
@@ -159,6 +161,7 @@ GINN_MAKE_SCALAR_FORWARDING_FACTORY(CwiseProd);
 // value = alpha * x + shift: ProdScalar (shift = 0) and AddScalar (alpha = 1).
 template <typename Scalar>
 class ScaleShiftNode : public BaseDataNode<Scalar> {
+ protected:
   NodePtr<Scalar> in_;
   float alpha_, shift_;
   const char* name_;
@@ -233,21 +236,181 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
 };
 GINN_MAKE_SCALAR_FORWARDING_FACTORY(CwiseProdAdd);
 
+// The scalar operand is held in the node's scalar type, as in the reference
+// (`val_(Scalar(b))`, ginn/node/common.h:45-46,218-219): for Half, x * 3.14
+// multiplies by the nearest Half.
 template <typename NodeT>
 auto ProdScalar(const Ptr<NodeT>& x, double a) {
   using Scalar = typename NodeT::Scalar;
-  return make_ptr<ScaleShiftNode<Scalar>>(NodePtr<Scalar>(x), static_cast<float>(a), 0.f, "ProdScalar");
+  return make_ptr<ScaleShiftNode<Scalar>>(NodePtr<Scalar>(x), static_cast<float>(Scalar(static_cast<float>(a))), 0.f,
+                                          "ProdScalar");
 }
 template <typename NodeT>
 auto AddScalar(const Ptr<NodeT>& x, double s) {
   using Scalar = typename NodeT::Scalar;
-  return make_ptr<ScaleShiftNode<Scalar>>(NodePtr<Scalar>(x), 1.f, static_cast<float>(s), "AddScalar");
+  return make_ptr<ScaleShiftNode<Scalar>>(NodePtr<Scalar>(x), 1.f, static_cast<float>(Scalar(static_cast<float>(s))),
+                                          "AddScalar");
+}
+// a - x for a scalar on the left (ginn/node/common.h:55-95).
+template <typename NodeT>
+auto SubtractScalar(double a, const Ptr<NodeT>& x) {
+  using Scalar = typename NodeT::Scalar;
+  return make_ptr<ScaleShiftNode<Scalar>>(NodePtr<Scalar>(x), -1.f, static_cast<float>(Scalar(static_cast<float>(a))),
+                                          "SubtractScalar");
 }
 
-template <typename Left, typename Right>
-auto operator+(const Ptr<Left>& a, const Ptr<Right>& b) {
-  using Scalar = typename Left::Scalar;
-  return Add(NodePtr<Scalar>(a), NodePtr<Scalar>(b));
+// value = left - right; backward left += dy, right -= dy (ginn/node/common.h:162-187).
+template <typename Scalar>
+class SubtractNode : public BaseDataNode<Scalar> {
+  NodePtr<Scalar> left_, right_;
+
+  void forward_() override {
+    internal::require_gpu(this->dev(), "Subtract");
+    GINN_ASSERT(left_->value().size() == right_->value().size(), "Subtract: operand sizes differ");
+    value().resize(left_->value().shape());
+    GINN_HIP_CALL(ginn_hip_elementwise(internal::ctx_of(value()), dtype_of<Scalar>(), GINN_HIP_EW_SUB,
+                                       static_cast<size_t>(value().size()), left_->value().data(),
+                                       right_->value().data(), nullptr, value().data(), 0));
+  }
+  void backward_() override {
+    if (left_->has_grad()) internal::add_tensors(left_->grad(), {&grad()}, true);
+    if (right_->has_grad())
+      GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(grad()), dtype_of<Scalar>(),
+                                         static_cast<size_t>(grad().size()), -1.f, 0.f, grad().data(),
+                                         right_->grad().data(), 1));
+  }
+
+ public:
+  using BaseDataNode<Scalar>::value;
+  using BaseDataNode<Scalar>::grad;
+  SubtractNode(const NodePtr<Scalar>& a, const NodePtr<Scalar>& b) : BaseDataNode<Scalar>({a, b}), left_(a), right_(b) {}
+  std::string name() const override { return "Subtract"; }
+};
+GINN_MAKE_SCALAR_FORWARDING_FACTORY(Subtract);
+
+// value = elementwise maximum of the inputs; the gradient goes to every input
+// that equals the maximum (ginn/node/common.h:319-357).
+template <typename Scalar>
+class CwiseMaxNode : public BaseDataNode<Scalar> {
+  std::vector<NodePtr<Scalar>> ins_;
+
+  void forward_() override {
+    internal::require_gpu(this->dev(), "CwiseMax");
+    value().resize(ins_[0]->value().shape());
+    value() = ins_[0]->value();
+    for (size_t i = 1; i < ins_.size(); ++i) {
+      GINN_ASSERT(ins_[i]->value().size() == value().size(), "CwiseMax: operand sizes differ");
+      GINN_HIP_CALL(ginn_hip_elementwise(internal::ctx_of(value()), dtype_of<Scalar>(), GINN_HIP_EW_MAX,
+                                         static_cast<size_t>(value().size()), value().data(),
+                                         ins_[i]->value().data(), nullptr, value().data(), 0));
+    }
+  }
+  void backward_() override {
+    for (auto& in : ins_)
+      if (in->has_grad())
+        GINN_HIP_CALL(ginn_hip_elementwise(internal::ctx_of(grad()), dtype_of<Scalar>(), GINN_HIP_EW_EQ_MUL,
+                                           static_cast<size_t>(grad().size()), grad().data(), in->value().data(),
+                                           value().data(), in->grad().data(), 1));
+  }
+
+ public:
+  using BaseDataNode<Scalar>::value;
+  using BaseDataNode<Scalar>::grad;
+  CwiseMaxNode(const std::vector<NodePtr<Scalar>>& ins) : BaseDataNode<Scalar>(ins), ins_(ins) {}
+  template <typename... Args>
+  CwiseMaxNode(const NodePtr<Scalar>& in, const Args&... args)
+      : CwiseMaxNode(std::vector<NodePtr<Scalar>>{in, args...}) {}
+  std::string name() const override { return "CwiseMax"; }
+};
+GINN_MAKE_SCALAR_FORWARDING_FACTORY(CwiseMax);
+
+// value = x * mask / (1 - p) with mask ~ Bernoulli(1 - p), drawn anew at every
+// forward pass (ginn/node/common.h:359-402).  The mask comes from a
+// counter-based generator on the device; seeds advance process-wide.
+template <typename Scalar>
+class DropoutNode : public BaseDataNode<Scalar> {
+  static_assert(is_floating_point_v<Scalar>, "Dropout scalar needs to be floating point because of scaling!");
+
+ protected:
+  NodePtr<Scalar> in_;
+  Real p_;
+  Tensor<bool> mask_;
+
+  static unsigned long long next_seed() {
+    static std::atomic<unsigned long long> s{0x2545f4914f6cdd1dull};
+    return s += 0x9e3779b97f4a7c15ull;
+  }
+  float scale() const { return static_cast<float>(Scalar(static_cast<float>(1. / (1. - p_)))); }
+
+  void forward_() override {
+    internal::require_gpu(this->dev(), "Dropout");
+    auto& x = in_->value();
+    value().resize(x.shape());
+    if (p_ == 1.) {
+      value().set_zero();
+      return;
+    }
+    mask_.resize(x.shape());
+    const size_t n = static_cast<size_t>(x.size());
+    GINN_HIP_CALL(ginn_hip_dropout_mask(internal::ctx_of(x), n, static_cast<float>(p_), next_seed(),
+                                        reinterpret_cast<unsigned char*>(mask_.data())));
+    GINN_HIP_CALL(ginn_hip_mask_scale(internal::ctx_of(x), dtype_of<Scalar>(), n, scale(), x.data(),
+                                      reinterpret_cast<const unsigned char*>(mask_.data()), value().data(), 0));
+  }
+  void backward_() override {
+    if (in_->has_grad() && p_ < 1.)
+      GINN_HIP_CALL(ginn_hip_mask_scale(internal::ctx_of(grad()), dtype_of<Scalar>(),
+                                        static_cast<size_t>(grad().size()), scale(), grad().data(),
+                                        reinterpret_cast<const unsigned char*>(mask_.data()), in_->grad().data(), 1));
+  }
+
+ public:
+  using BaseDataNode<Scalar>::value;
+  using BaseDataNode<Scalar>::grad;
+  DropoutNode(const NodePtr<Scalar>& in, Real p)
+      : BaseDataNode<Scalar>(std::vector<BaseNodePtr>{in}), in_(in), p_(p), mask_(in->dev()) {
+    GINN_ASSERT(p_ >= 0 && p_ <= 1, "Dropout probability is not in [0, 1]!");
+  }
+  const Tensor<bool>& mask() const { return mask_; }
+  std::string name() const override { return "Dropout"; }
+};
+GINN_MAKE_SCALAR_FORWARDING_FACTORY(Dropout);
+
+// Operator sugar (ginn/node/common.h:404-479): node (+|-) node, node (+|-|*) scalar,
+// scalar (+|-|*) node, -node.
+template <typename Left, typename Right,
+          typename = std::enable_if_t<is_node_ptr_v<Left> || is_node_ptr_v<Right>>>
+auto operator+(const Left& a, const Right& b) {
+  if constexpr (is_node_ptr_v<Left> && is_node_ptr_v<Right>) {
+    using Scalar = typename Left::element_type::Scalar;
+    return Add(NodePtr<Scalar>(a), NodePtr<Scalar>(b));
+  } else if constexpr (is_node_ptr_v<Left>) {
+    return AddScalar(a, static_cast<double>(b));
+  } else {
+    return AddScalar(b, static_cast<double>(a));
+  }
+}
+template <typename Left, typename Right,
+          typename = std::enable_if_t<is_node_ptr_v<Left> || is_node_ptr_v<Right>>>
+auto operator-(const Left& a, const Right& b) {
+  if constexpr (is_node_ptr_v<Left> && is_node_ptr_v<Right>) {
+    using Scalar = typename Left::element_type::Scalar;
+    return Subtract(NodePtr<Scalar>(a), NodePtr<Scalar>(b));
+  } else if constexpr (is_node_ptr_v<Left>) {
+    return AddScalar(a, -static_cast<double>(b));
+  } else {
+    return SubtractScalar(static_cast<double>(a), b);
+  }
+}
+template <typename NodeT>
+auto operator-(const Ptr<NodeT>& in) {
+  return ProdScalar(in, -1.);
+}
+template <typename Left, typename Right,
+          typename = std::enable_if_t<is_node_ptr_v<Left> != is_node_ptr_v<Right>>>
+auto operator*(const Left& a, const Right& b) {
+  if constexpr (is_node_ptr_v<Left>) return ProdScalar(a, static_cast<double>(b));
+  else return ProdScalar(b, static_cast<double>(a));
 }
 
 }  // namespace ginn

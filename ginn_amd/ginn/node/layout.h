@@ -466,8 +466,28 @@ GINN_MAKE_SCALAR_FORWARDING_FACTORY(Map);
 // (ginn/node/layout.h:723-821); backward adds the inversely permuted gradient.
 template <typename Scalar>
 class PermuteNode : public BaseDataNode<Scalar> {
+ protected:
   NodePtr<Scalar> in_;
   Shape indices_;
+  bool overwrite_ = false;  // set by InPlacePermuteNode: results replace, through a temporary
+
+  static Shape permute(const Shape& s, const Shape& perm) {
+    Shape out(s.size());
+    for (size_t i = 0; i < s.size(); ++i) out[i] = s[static_cast<size_t>(perm[i])];
+    return out;
+  }
+  static Shape inverse(const Shape& perm) {
+    Shape inv(perm.size());
+    for (size_t i = 0; i < perm.size(); ++i) inv[static_cast<size_t>(perm[i])] = static_cast<Size>(i);
+    return inv;
+  }
+  void check_permutation(const Shape& s) const {
+    GINN_ASSERT(indices_.size() == s.size());
+    Shape seen(s.size(), 0);
+    for (Size i : indices_)
+      GINN_ASSERT(i >= 0 && i < static_cast<Size>(s.size()) && !seen[static_cast<size_t>(i)]++,
+                  "Indices are not a proper permutation in Permute!");
+  }
 
   static void run(const Tensor<Scalar>& src, const Shape& src_shape, const Shape& perm, Tensor<Scalar>& dst,
                   bool accumulate) {
@@ -479,21 +499,23 @@ class PermuteNode : public BaseDataNode<Scalar> {
   }
   void forward_() override {
     const Shape s = in_->value().shape();
-    GINN_ASSERT(indices_.size() == s.size());
-    Shape seen(s.size(), 0), out(s.size());
-    for (size_t i = 0; i < s.size(); ++i) {
-      GINN_ASSERT(indices_[i] >= 0 && indices_[i] < static_cast<Size>(s.size()) && !seen[indices_[i]]++,
-                  "Indices are not a proper permutation in Permute!");
-      out[i] = s[indices_[i]];
-    }
-    value().resize(out);
+    check_permutation(s);
+    value().resize(permute(s, indices_));
     run(in_->value(), s, indices_, value(), false);
   }
   void backward_() override {
     if (!in_->has_grad()) return;
-    Shape inv(indices_.size());
-    for (size_t i = 0; i < indices_.size(); ++i) inv[indices_[i]] = static_cast<Size>(i);
-    run(grad(), grad().shape(), inv, in_->grad(), true);
+    if (overwrite_) {
+      // grad() is in's gradient storage under the permuted shape: permute into a
+      // temporary and copy back (the reference's `.eval()`, ginn/node/layout.h:766-770).
+      Tensor<Scalar> tmp(grad().dev(), in_->shape());
+      run(grad(), grad().shape(), inverse(indices_), tmp, false);
+      Tensor<Scalar> flat;
+      flat.map(in_->grad(), in_->shape());
+      flat = tmp;
+    } else {
+      run(grad(), grad().shape(), inverse(indices_), in_->grad(), true);
+    }
   }
 
  public:
@@ -504,6 +526,171 @@ class PermuteNode : public BaseDataNode<Scalar> {
   std::string name() const override { return "Permute"; }
 };
 GINN_MAKE_SCALAR_FORWARDING_FACTORY(Permute);
+
+template <typename NodePtrType>
+auto Permute(NodePtrType x, std::initializer_list<Size> indices) {
+  return Permute(std::move(x), Shape(indices));
+}
+
+// Swaps two axes (ginn/node/layout.h:822-828).
+template <typename NodePtrType>
+auto Transpose(NodePtrType x, Size i, Size j) {
+  Shape indices(x->shape().size());
+  std::iota(indices.begin(), indices.end(), Size(0));
+  std::swap(indices.at(static_cast<size_t>(i)), indices.at(static_cast<size_t>(j)));
+  return Permute(std::move(x), std::move(indices));
+}
+
+// The sub-tensor at position `offset` of axis `dim`; the result has one axis
+// less (ginn/node/layout.h:631-697).  With the input viewed as
+// [inner, extent(dim), outer] this is a strided copy.
+template <typename Scalar>
+class ChipNode : public BaseDataNode<Scalar> {
+  NodePtr<Scalar> in_;
+  Size offset_, dim_;
+
+  void geometry(Size& inner, Size& extent, Size& outer) const {
+    const Shape s = in_->shape();
+    inner = outer = 1;
+    for (Size a = 0; a < dim_; ++a) inner *= s[static_cast<size_t>(a)];
+    extent = s[static_cast<size_t>(dim_)];
+    for (size_t a = static_cast<size_t>(dim_) + 1; a < s.size(); ++a) outer *= s[a];
+  }
+  void forward_() override {
+    internal::require_gpu(this->dev(), "Chip");
+    const Shape in_s = in_->shape();
+    GINN_ASSERT(dim_ >= 0 && static_cast<size_t>(dim_) < in_s.size());
+    GINN_ASSERT(offset_ >= 0 && offset_ < in_s[static_cast<size_t>(dim_)]);
+    GINN_ASSERT(in_s.size() >= 2 && in_s.size() <= 8, "Unexpected input rank in Chip!");
+    Shape s = in_s;
+    s.erase(s.begin() + dim_);
+    value().resize(s);
+    Size inner, extent, outer;
+    geometry(inner, extent, outer);
+    GINN_HIP_CALL(ginn_hip_copy_2d(internal::ctx_of(value()), dtype_of<Scalar>(), static_cast<int>(inner),
+                                   static_cast<int>(outer), in_->value().data() + offset_ * inner,
+                                   static_cast<int>(inner * extent), value().data(), static_cast<int>(inner), 0));
+  }
+  void backward_() override {
+    if (!in_->has_grad()) return;
+    Size inner, extent, outer;
+    geometry(inner, extent, outer);
+    GINN_HIP_CALL(ginn_hip_copy_2d(internal::ctx_of(grad()), dtype_of<Scalar>(), static_cast<int>(inner),
+                                   static_cast<int>(outer), grad().data(), static_cast<int>(inner),
+                                   in_->grad().data() + offset_ * inner, static_cast<int>(inner * extent), 1));
+  }
+
+ public:
+  using BaseDataNode<Scalar>::value;
+  using BaseDataNode<Scalar>::grad;
+  ChipNode(const NodePtr<Scalar>& x, Size offset, Size dim) : BaseDataNode<Scalar>({x}), in_(x), offset_(offset), dim_(dim) {}
+  std::string name() const override { return "Chip"; }
+};
+GINN_MAKE_SCALAR_FORWARDING_FACTORY(Chip);
+
+// An m x n grid of equally shaped tensors as one tensor of shape
+// (their shape) + {m, n}: embedding lookups stacked into a batch
+// (ginn/node/layout.h:350-466).  One gather kernel over a device table of the
+// inputs' addresses; backward adds atomically, because a grid may hold one
+// node in several places.
+template <typename Scalar>
+class StackNode : public BaseDataNode<Scalar> {
+  std::vector<std::vector<NodePtr<Scalar>>> nodes_;
+  Tensor<void*> table_;  // device copy of the address table of the pass under way
+
+  static std::vector<BaseNodePtr> flatten(const std::vector<std::vector<NodePtr<Scalar>>>& nodes) {
+    std::vector<BaseNodePtr> flat;
+    for (auto& inner : nodes)
+      for (auto& x : inner) flat.push_back(x);
+    return flat;
+  }
+  // Entry j * m + i names what nodes_[i][j] yields through `get` (NULL allowed).
+  template <typename Get>
+  void* upload_table(Get get) {
+    const size_t m = nodes_.size(), n = nodes_[0].size();
+    std::vector<void*> host(m * n);
+    for (size_t i = 0; i < m; ++i)
+      for (size_t j = 0; j < n; ++j) host[j * m + i] = get(nodes_[i][j]);
+    table_.move_to(this->dev());
+    table_.resize({static_cast<Size>(host.size())});
+    table_.set(host);
+    return table_.data();
+  }
+  void forward_() override {
+    internal::require_gpu(this->dev(), "Stack");
+    const Size m = static_cast<Size>(nodes_.size()), n = static_cast<Size>(nodes_[0].size());
+    const Shape s = nodes_[0][0]->shape();
+    for (auto& inner : nodes_)
+      for (auto& x : inner) GINN_ASSERT(x->shape() == s, "Input shapes mismatch!");
+    Shape ns = s;
+    ns.push_back(m);
+    ns.push_back(n);
+    value().resize(ns);
+    const size_t sz = static_cast<size_t>(nodes_[0][0]->size());
+    void* table = upload_table([](const NodePtr<Scalar>& x) { return static_cast<void*>(x->value().data()); });
+    GINN_HIP_CALL(ginn_hip_stack(internal::ctx_of(value()), static_cast<int>(sizeof(Scalar)), sz,
+                                 static_cast<size_t>(m * n), static_cast<const void* const*>(table), value().data()));
+  }
+  void backward_() override {
+    if constexpr (is_floating_point_v<Scalar>) {
+      const size_t sz = static_cast<size_t>(nodes_[0][0]->size());
+      void* table = upload_table([](const NodePtr<Scalar>& x) {
+        return x->has_grad() ? static_cast<void*>(x->grad().data()) : nullptr;
+      });
+      GINN_HIP_CALL(ginn_hip_stack_bwd(internal::ctx_of(grad()), dtype_of<Scalar>(), sz,
+                                       nodes_.size() * nodes_[0].size(), static_cast<void* const*>(table),
+                                       grad().data()));
+    }
+  }
+
+ public:
+  using BaseDataNode<Scalar>::value;
+  using BaseDataNode<Scalar>::grad;
+  StackNode(const std::vector<std::vector<NodePtr<Scalar>>>& nodes)
+      : BaseDataNode<Scalar>(flatten(nodes)), nodes_(nodes) {
+    GINN_ASSERT(!nodes_.empty(), "Empty input to Stack!");
+    GINN_ASSERT(!nodes_.front().empty(), "Empty input to Stack!");
+    for (auto& inner : nodes_) GINN_ASSERT(inner.size() == nodes_.front().size(), "Inner container sizes mismatch!");
+  }
+  std::string name() const override { return "Stack"; }
+};
+template <typename Scalar>
+auto Stack(const std::vector<std::vector<NodePtr<Scalar>>>& ins) {
+  return make_ptr<StackNode<Scalar>>(ins);
+}
+
+// A [1 x cols] row repeated `rows` times; backward sums the gradient over the
+// rows (ginn/node/layout.h:831-862).
+template <typename Scalar>
+class RowBroadcastNode : public BaseDataNode<Scalar> {
+  NodePtr<Scalar> in_;
+  DimPtr rows_;
+
+  void forward_() override {
+    internal::require_gpu(this->dev(), "RowBroadcast");
+    auto& x = in_->value();
+    GINN_ASSERT(x.shape().size() == 2);
+    GINN_ASSERT(x.rows() == 1);
+    const Size rows = rows_->value();
+    value().resize(rows, x.cols());
+    GINN_HIP_CALL(ginn_hip_row_broadcast(internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(rows),
+                                         static_cast<int>(x.cols()), x.data(), value().data()));
+  }
+  void backward_() override {
+    if (in_->has_grad())
+      GINN_HIP_CALL(ginn_hip_col_sum(internal::ctx_of(grad()), dtype_of<Scalar>(), static_cast<int>(grad().rows()),
+                                     static_cast<int>(grad().cols()), grad().data(), in_->grad().data(), 1));
+  }
+
+ public:
+  using BaseDataNode<Scalar>::value;
+  using BaseDataNode<Scalar>::grad;
+  RowBroadcastNode(const NodePtr<Scalar>& in, DimPtr rows)
+      : BaseDataNode<Scalar>(std::vector<BaseNodePtr>{in, rows}), in_(in), rows_(rows) {}
+  RowBroadcastNode(const NodePtr<Scalar>& in, Size rows) : RowBroadcastNode(in, make_ptr<DimNode>(rows)) {}
+  std::string name() const override { return "RowBroadcast"; }
+};
+GINN_MAKE_SCALAR_FORWARDING_FACTORY(RowBroadcast);
 
 // Square matrix of ones on and above the diagonal, zeros below: the causal
 // attention mask (ginn/node/layout.h:922-955).  Carries no gradient.

@@ -249,7 +249,14 @@ class Tensor {
   // Copy of the elements in storage order, from any device.
   std::vector<Scalar> vector() const {
     std::vector<Scalar> out(static_cast<size_t>(size()));
-    if (size() > 0) cpu()->copy(*dev_, out.data(), data_, out.size() * sizeof(Scalar));
+    if (size() == 0) return out;
+    if constexpr (std::is_same_v<Scalar, bool>) {  // std::vector<bool> is packed: go through bytes
+      std::vector<unsigned char> bytes(out.size());
+      cpu()->copy(*dev_, bytes.data(), data_, bytes.size());
+      for (size_t i = 0; i < out.size(); ++i) out[i] = bytes[i] != 0;
+    } else {
+      cpu()->copy(*dev_, out.data(), data_, out.size() * sizeof(Scalar));
+    }
     return out;
   }
   Scalar item() const {
@@ -284,9 +291,11 @@ class Tensor {
   }
   void set_ones() { fill(Scalar(1)); }
 
-  // Uniform in [-1, 1) (ginn/tensor.h:455-462).  The reference's stream comes
-  // from Eigen / cuRAND; this one is a SplitMix64 counter stream, generated on
-  // the host so that host and device copies of a tensor agree.
+  // Uniform in [-1, 1) (ginn/tensor.h:446-470).  The reference's streams come
+  // from Eigen (host) and cuRAND (device); here a host tensor draws from a
+  // SplitMix64 counter stream and a floating-point device tensor is filled on
+  // the device from (seed, element index), the seed advancing per call; other
+  // device tensors are drawn on the host and copied.
   static uint64_t& random_state() {
     static uint64_t s = 0x9e3779b97f4a7c15ull;
     return s;
@@ -294,6 +303,15 @@ class Tensor {
   static void seed(uint64_t s) { random_state() = s * 0x9e3779b97f4a7c15ull + 0x632be59bd9b4e019ull; }
   void set_random() {
     if (size() == 0) return;
+    if constexpr (is_floating_point_v<Scalar>) {
+      if (dev_->kind() == GPU) {
+        uint64_t& s = random_state();
+        s += 0x9e3779b97f4a7c15ull;
+        GINN_HIP_CALL(ginn_hip_fill_uniform(ctx(), dtype_of<Scalar>(), static_cast<size_t>(size()), s, -1.f, 1.f,
+                                            data_));
+        return;
+      }
+    }
     std::vector<Scalar> host(static_cast<size_t>(size()));
     uint64_t& s = random_state();
     for (auto& x : host) {
@@ -311,8 +329,14 @@ class Tensor {
   // Values in storage (column-major) order.
   void set(const std::vector<Scalar>& vals) {
     GINN_ASSERT(static_cast<Size>(vals.size()) == size());
-    if (size() > 0)
+    if (size() == 0) return;
+    if constexpr (std::is_same_v<Scalar, bool>) {
+      std::vector<unsigned char> bytes(vals.size());
+      for (size_t i = 0; i < vals.size(); ++i) bytes[i] = vals[i] ? 1 : 0;
+      dev_->copy(*cpu(), data_, bytes.data(), bytes.size());
+    } else {
       dev_->copy(*cpu(), data_, const_cast<Scalar*>(vals.data()), vals.size() * sizeof(Scalar));
+    }
   }
 
   // The first min(size(), vals.size()) elements, converted (ginn/tensor.h:472-489).

@@ -42,7 +42,10 @@ typedef struct ginn_hip_arena ginn_hip_arena;
 typedef enum ginn_hip_dtype {
   GINN_HIP_F32 = 0,
   GINN_HIP_F16 = 1,
-  GINN_HIP_BF16 = 2
+  GINN_HIP_BF16 = 2,
+  /* ginn::Int index tensors: accepted only where a declaration says so
+   * (comparison); no arithmetic entry point takes it. */
+  GINN_HIP_I32 = 3
 } ginn_hip_dtype;
 
 /* CUBLAS_OP_N / CUBLAS_OP_T as used by ginn/prod.h:217-222. */
@@ -399,6 +402,135 @@ int ginn_hip_mask_fill(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
  * row <= col, else 0. */
 int ginn_hip_upper_tri(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int n,
                        void* dst);
+
+/* LayerNormNode::backward_ of the in-place node (ginn/node/inplace.h:214-246):
+ * dx = (...) / std, assigned; dx may be dy itself. */
+int ginn_hip_layernorm_bwd_assign(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                                  int rows, int cols, const void* dy,
+                                  const void* y, const float* std_in, void* dx);
+
+/* ------------------------------------------------------------------ */
+/* The other nodes around the products: arithmetic, selection, gather  */
+/* / scatter, reductions, random fills.  Eigen expressions, thrust      */
+/* gathers and the two Stack kernels in the reference.                  */
+/* ------------------------------------------------------------------ */
+
+typedef enum {
+  GINN_HIP_EW_SUB = 0,    /* a - b                 SubtractNode forward (ginn/node/common.h:162-187) */
+  GINN_HIP_EW_MAX = 1,    /* max(a, b)             CwiseMaxNode forward, pairwise (:319-330) */
+  GINN_HIP_EW_EQ_MUL = 2, /* a * (b == c ? 1 : 0)  CwiseMaxNode backward (:332-341) */
+  GINN_HIP_EW_DIV_MUL = 3 /* a * (b / c)           InPlaceCwiseProdNode backward (ginn/node/inplace.h:88-93) */
+} ginn_hip_ew_op;
+
+/* dst (+)= op(a, b, c) over n elements; c is read by the three-operand forms
+ * only.  dst may be one of the operands. */
+int ginn_hip_elementwise(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                         ginn_hip_ew_op op, size_t n, const void* a,
+                         const void* b, const void* c, void* dst,
+                         int accumulate);
+
+/* U[lo, hi) fill: element i is a function of (seed, i) alone.  Replaces
+ * curandGenerateUniform + `-1 + 2 x` of Tensor::set_random on a GPU tensor
+ * (ginn/tensor.h:459-462, ginn/cudef.h:63-89); the value stream differs from
+ * cuRAND's, as cuRAND's differs from Eigen's. */
+int ginn_hip_fill_uniform(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
+                          unsigned long long seed, float lo, float hi,
+                          void* dst);
+
+/* DropoutNode (ginn/node/common.h:359-402): mask[i] = (u_i >= p), one byte
+ * per element, u_i uniform in [0, 1) from (seed, i); then
+ * dst (+)= x * mask * scale with scale = 1 / (1 - p) serves the forward pass
+ * and, on the gradient, the backward pass (dst may be x: InPlaceDropout,
+ * ginn/node/inplace.h:126-150). */
+int ginn_hip_dropout_mask(ginn_hip_ctx* ctx, size_t n, float p,
+                          unsigned long long seed, unsigned char* mask);
+int ginn_hip_mask_scale(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
+                        float scale, const void* x, const unsigned char* mask,
+                        void* dst, int accumulate);
+
+/* SelectNode (ginn/node/select.h:24-112): dst[i] = cond[i] ? a : b, cond one
+ * byte per element (Tensor<bool>); a branch flagged scalar is a single value
+ * used for every i.  Backward: dst[i] += dy[i] where (cond[i] != 0) == want,
+ * summed into dst[0] when the branch is a single value. */
+int ginn_hip_select(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
+                    const unsigned char* cond, const void* a, int a_is_scalar,
+                    const void* b, int b_is_scalar, void* dst);
+int ginn_hip_select_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
+                        const unsigned char* cond, int want, const void* dy,
+                        void* dst, int dst_is_scalar);
+
+/* MaskNode (ginn/node/select.h:114-187): x viewed as [mask_size x batch];
+ * dst (+)= mask != 0 ? x : value.  Forward with `value` = the mask value,
+ * backward on the gradient with value 0 and accumulate. */
+int ginn_hip_mask_select(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                         size_t mask_size, size_t batch, const void* mask,
+                         float value, const void* x, void* dst, int accumulate);
+
+/* LessThanNode (ginn/node/compare.h:27-56): out[i] = a[i] < b[i], one byte
+ * each; dtype may be GINN_HIP_I32. */
+int ginn_hip_less_than(ginn_hip_ctx* ctx, int dtype, size_t n, const void* a,
+                       const void* b, unsigned char* out);
+
+/* PickNode (ginn/node/pick.h:29-170): out[c] = x[idx[c], c] for a [rows x cols]
+ * x (thrust::gather in the reference); backward dx[idx[c], c] += sign * dout[c]
+ * (its gather + add + scatter).  An index outside [0, rows) picks NaN and
+ * receives nothing. */
+int ginn_hip_pick(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols,
+                  const void* x, const int* idx, void* out);
+int ginn_hip_pick_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows,
+                      int cols, const int* idx, const void* dout, float sign,
+                      void* dx);
+
+/* PickNegLogSigmoidNode (ginn/node/pick.h:250-304): sigm = sigmoid(x),
+ * out = -(idx ? log sigm : log(1 - sigm)) elementwise, idx int32 of the same
+ * shape; backward dx += (sigm - idx) * dout. */
+int ginn_hip_pick_nlsig_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
+                            const void* x, const int* idx, void* sigm,
+                            void* out);
+int ginn_hip_pick_nlsig_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
+                            const void* sigm, const int* idx, const void* dout,
+                            void* dx);
+
+/* AxisSumNode (ginn/node/reduce.h:53-136): sums x over the axes flagged in
+ * host_summed (HOST arrays of `rank` <= 8 entries); dst holds the remaining
+ * axes in order.  Backward: dx[i] += dy[i projected onto the kept axes]. */
+int ginn_hip_axis_sum(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rank,
+                      const long long* host_dims, const int* host_summed,
+                      const void* x, void* dst);
+int ginn_hip_axis_sum_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rank,
+                          const long long* host_dims, const int* host_summed,
+                          const void* dy, void* dx);
+
+/* VarianceNode (ginn/node/reduce.h:164-204): mean_out[0] = mean(x),
+ * var_out[0] = mean((x - mean)^2); backward dx += (x - mean) * dvar * 2 / n. */
+int ginn_hip_variance_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
+                          const void* x, void* mean_out, void* var_out);
+int ginn_hip_variance_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
+                          const void* x, const void* mean, const void* dvar,
+                          void* dx);
+
+/* StackNode (ginn/node/layout.h:324-444): dst = the `count` arrays of `sz`
+ * elements named by the DEVICE table dev_srcs, one after the other
+ * (stack_helper); elements of 1, 2 or 4 bytes.  Backward: array k receives
+ * src[k * sz ...] added atomically (stack_backward_helper; a table may name
+ * an array several times); NULL entries are inputs without gradient. */
+int ginn_hip_stack(ginn_hip_ctx* ctx, int elem_bytes, size_t sz, size_t count,
+                   const void* const* dev_srcs, void* dst);
+int ginn_hip_stack_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t sz,
+                       size_t count, void* const* dev_dsts, const void* src);
+
+/* argmax (ginn/util/amax.h:28-66) along the middle axis of x viewed as
+ * [inner x len x outer]: out[inner x outer] int64 positions, the first
+ * maximum wins. */
+int ginn_hip_argmax(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t inner,
+                    size_t len, size_t outer, const void* x, long long* out);
+
+/* RowBroadcastNode (ginn/node/layout.h:831-862): dst[r, c] = x[c]; its
+ * backward is the column sum dst[c] (+)= sum_r x[r, c]. */
+int ginn_hip_row_broadcast(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows,
+                           int cols, const void* x, void* dst);
+int ginn_hip_col_sum(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows,
+                     int cols, const void* x, void* dst, int accumulate);
 
 /* ------------------------------------------------------------------ */
 /* Many elementwise operations in one launch                            */
