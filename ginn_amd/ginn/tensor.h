@@ -274,8 +274,7 @@ class Tensor {
         GINN_HIP_CALL(ginn_hip_fill(ctx(), dtype_of<Scalar>(), data_, static_cast<size_t>(size()),
                                     static_cast<float>(val)));
       } else {
-        std::vector<Scalar> host(static_cast<size_t>(size()), val);
-        dev_->copy(*cpu(), data_, host.data(), host.size() * sizeof(Scalar));
+        set(std::vector<Scalar>(static_cast<size_t>(size()), val));
       }
     } else {
       GINN_THROW("Unexpected device in Tensor::fill!");
@@ -314,16 +313,16 @@ class Tensor {
     }
     std::vector<Scalar> host(static_cast<size_t>(size()));
     uint64_t& s = random_state();
-    for (auto& x : host) {
+    for (size_t i = 0; i < host.size(); ++i) {
       s += 0x9e3779b97f4a7c15ull;
       uint64_t z = s;
       z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
       z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
       z ^= z >> 31;
       const double u = static_cast<double>(z >> 11) * (1.0 / 9007199254740992.0);
-      x = Scalar(static_cast<float>(2.0 * u - 1.0));
+      host[i] = Scalar(static_cast<float>(2.0 * u - 1.0));
     }
-    dev_->copy(*cpu(), data_, host.data(), host.size() * sizeof(Scalar));
+    set(host);
   }
 
   // Values in storage (column-major) order.
@@ -433,11 +432,11 @@ class Tensor {
     for (Size& dim : new_shape) in >> dim;
     resize(new_shape);
     std::vector<Scalar> vals(static_cast<size_t>(size()));
-    for (auto& x : vals) {
+    for (size_t i = 0; i < vals.size(); ++i) {
       double val = 0;
       in >> val;
-      if constexpr (is_floating_point_v<Scalar>) x = Scalar(static_cast<float>(val));
-      else x = static_cast<Scalar>(val);
+      if constexpr (is_floating_point_v<Scalar>) vals[i] = Scalar(static_cast<float>(val));
+      else vals[i] = static_cast<Scalar>(val);
     }
     GINN_ASSERT(!in.fail(), "Tensor::load: malformed or truncated element list");
     char end_of_line = 0;

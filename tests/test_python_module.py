@@ -160,3 +160,132 @@ def test_prod_nodes_and_autobatch_from_python(ginn):
         ex.forward()
         assert abs(g2.sink.value.list()[0] - plain) <= 1e-5 * max(1.0, abs(plain))
         assert g2.size != g.size
+
+
+def test_scalars_tensors_and_casts(ginn):
+    """Every scalar of ginn-py/tensor-py.h:36-48 (plus BFloat16): tensors exchange
+    values with numpy, a Real data node casts to each of them."""
+    a = np.array([[1.5, -2.0], [0.25, 4.0]])
+    for name, cls in (("Half", ginn.HalfTensor), ("BFloat16", ginn.BFloat16Tensor)):
+        t = cls(ginn.cpu(), [1])
+        t.set(a)
+        assert t.shape == [2, 2] and t.scalar == getattr(ginn, name)
+        np.testing.assert_array_equal(np.asarray(t.numpy(), dtype=np.float64), a)  # exactly representable
+    assert ginn.HalfTensor(ginn.cpu(), [2]).numpy().dtype == np.float16
+    b = ginn.BoolTensor(ginn.cpu(), [1])
+    b.set(np.array([[True, False], [False, True]]))
+    assert b.list() == [True, False, False, True]
+    x = ginn.Values(ginn.cpu(), [[1, 2, 3], [4, 5, 6]])
+    assert x.shape == [2, 3] and x.value.list() == [1, 4, 2, 5, 3, 6]
+    for scalar, cls in ((ginn.Real, "RealDataNode"), (ginn.Half, "HalfDataNode"), (ginn.BFloat16, "BFloat16DataNode"),
+                        (ginn.Int, "IntDataNode"), (ginn.Bool, "BoolDataNode")):
+        y = x.cast(scalar)
+        assert type(y).__name__ == cls and y.shape == [2, 3]
+        assert [float(v) for v in y.value.list()] == ([1.0] * 6 if scalar == ginn.Bool else [1, 4, 2, 5, 3, 6])
+    w = ginn.Weight(scalar=ginn.Half, device=ginn.cpu(), shape=[2, 3])
+    assert type(w).__name__ == "HalfWeightNode" and w.forwarded
+    w.reset_forwarded()
+    assert w.forwarded  # weights stay forwarded (ginn-py/test/test_nodes.py:945-948)
+    w2 = w.copy(ginn.Copy.Tied)
+    assert w2.id == w.id
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("scalar_name", ["Real", "Half", "BFloat16"])
+def test_reference_python_cases(ginn, scalar_name):
+    """test_prod, test_batched_prod, test_affine, test_affine_w_broadcast and
+    test_affine_w_high_rank of ginn-py/test/test_nodes.py:804-936, on the device,
+    for Real and Half as there (Half eps 1e-2 / 2e-3) and for BFloat16."""
+    scalar = getattr(ginn, scalar_name)
+    dev = ginn.gpu()
+    eps = {"Real": 1e-6, "Half": 1e-2, "BFloat16": 3e-2}[scalar_name]
+
+    def check(a, b, eps):
+        ginn.Graph(a).forward()
+        ginn.Graph(b).forward()
+        a_, b_ = a.value.maybe_copy_to(ginn.cpu()), b.value.maybe_copy_to(ginn.cpu())
+        assert a_.shape == b_.shape
+        assert a_.list() == pytest.approx(b_.list(), rel=eps, abs=eps * 1e-2)
+
+    W = ginn.Values(dev, [[1, 2, 3], [4, 5, 6]]).cast(scalar)
+    V = ginn.Values(dev, [[0.6, 0.5], [0.4, -0.1], [-0.2, -0.3]]).cast(scalar)
+    WV = ginn.Values(dev, [[0.8, -0.6], [3.2, -0.3]]).cast(scalar)
+    check(ginn.Prod(W, V), WV, eps)
+    check(W * V, WV, eps)
+
+    a = ginn.Random(dev, [2, 3, 4]).cast(scalar)
+    b = ginn.Random(dev, [3, 5, 4]).cast(scalar)
+    c = ginn.BatchedProd(a, b)
+    for i in range(4):
+        check(ginn.Chip(c, i, 2), ginn.Chip(a, i, 2) * ginn.Chip(b, i, 2), max(eps, 1e-5))
+
+    Vc = ginn.Values(dev, [[0.6], [0.4], [-0.2]]).cast(scalar)
+    bias = ginn.Values(dev, [[0.01], [0.02]]).cast(scalar)
+    WVb = ginn.Values(dev, [[0.81], [3.22]]).cast(scalar)
+    aeps = {"Real": 1e-6, "Half": 2e-3, "BFloat16": 2e-2}[scalar_name]
+    check(ginn.Affine([W, Vc, bias]), WVb, aeps)
+    check(W * Vc + bias, WVb, aeps)
+    V2 = ginn.Values(dev, [[6, 5], [4, -1], [-2, -3]]).cast(scalar)
+    b2 = ginn.Values(dev, [[0.1], [0.2]]).cast(scalar)
+    check(ginn.Affine([W, V2, b2]), ginn.Values(dev, [[8.1, -5.9], [32.2, -2.8]]).cast(scalar), aeps)
+    V3 = ginn.Values(dev, [[[6, 5], [6, 5]], [[4, -1], [4, -1]], [[-2, -3], [-2, -3]]]).cast(scalar)
+    want = ginn.Values(dev, [[[8.1, -5.9], [8.1, -5.9]], [[32.2, -2.8], [32.2, -2.8]]]).cast(scalar)
+    check(ginn.Affine([W, V3, b2]), want, aeps)
+    # a few of the other nodes through the bindings
+    check(ginn.AxisSum(V3, [0, 2]), ginn.Values(dev, [9.0, 9.0]).cast(scalar), aeps)
+    check(1 - W, ginn.Values(dev, [[0, -1, -2], [-3, -4, -5]]).cast(scalar), aeps)
+    lt = W < (W * 0 + 3.5)
+    ginn.Graph(lt).forward()
+    assert lt.value.list() == [True, False, True, False, True, False]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("scalar_name", ["Half", "BFloat16"])
+def test_mnist_style_training_loop_16bit(ginn, scalar_name):
+    """The loop of ginn-py/examples/mnist.py:62-92 with 16-bit weights and
+    activations (fp32 accumulation in the products): losses, gradients and
+    weights follow the oracle within the 16-bit tolerance.  Plain gradient
+    steps: Adam's step is +-lr whatever the size of a gradient, so an entry whose
+    gradient is below the 16-bit rounding may legitimately move the other way."""
+    from oracle import nodes as N
+    from oracle import update as U
+    scalar = getattr(ginn, scalar_name)
+    rng = np.random.default_rng(11)
+    dimx, dimh, dimy, bs, lr = 64, 48, 10, 16, 1e-2
+    dev = ginn.gpu()
+    shapes = [[dimh, dimx], [dimh], [dimy, dimh], [dimy]]
+    weights = [ginn.Weight(dev, s, scalar) for s in shapes]
+    host = []
+    for w, s in zip(weights, shapes):
+        w.value.set(rng.uniform(-0.3, 0.3, s))
+        host.append(np.asarray(w.value.numpy(), dtype=np.float64))  # the values as stored
+    W, b, V, c = weights
+    x_np = rng.uniform(0, 1, (dimx, bs))
+    y_np = rng.integers(0, dimy, (1, bs))
+    x = ginn.Data(x_np)
+    x.move_to(dev)
+    xs = x.cast(scalar)
+    x_np = np.asarray(xs.value.numpy(), dtype=np.float64)
+    y = ginn.Data(y_np.astype(np.float32)).int()
+    y.move_to(dev)
+    assert type(ginn.Adam(lr, scalar=scalar)).__name__ == scalar_name + "Adam"
+    updater = ginn.Sgd(0.1, 5.0, scalar=scalar)
+    ref = [h.astype(np.float32) for h in host]
+    for step in range(3):
+        h = ginn.Sigmoid(ginn.Affine([W, xs, b]))
+        loss = ginn.Sum(ginn.PickNegLogSoftmax(ginn.Affine([V, h, c]), y))
+        g = ginn.Graph(loss)
+        g.forward()
+        g.reset_grad()
+        g.backward(1.0)
+        want_loss, _, dWs, dbs = N.mlp_forward_backward(
+            [N.SIGMOID, N.IDENTITY], [ref[0].astype(np.float64), ref[2].astype(np.float64)],
+            [ref[1].astype(np.float64), ref[3].astype(np.float64)], x_np, y_np.reshape(-1).astype(np.int32))
+        assert abs(loss.value.list()[0] - want_loss) <= 2e-2 * abs(want_loss)
+        assert rel_fro(np.asarray(W.grad.numpy(), np.float64), dWs[0]) <= 2e-2
+        assert rel_fro(np.asarray(V.grad.numpy(), np.float64), dWs[1]) <= 2e-2
+        updater.update(weights)
+        for i, grad in enumerate([dWs[0], dbs[0], dWs[1], dbs[1]]):
+            ref[i], _ = U.sgd_update(ref[i], grad.astype(np.float32).reshape(ref[i].shape), lr=0.1)
+    for w, r in zip(weights, ref):
+        assert rel_fro(np.asarray(w.value.numpy(), np.float64), r) <= 2e-2
