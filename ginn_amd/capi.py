@@ -32,6 +32,9 @@ PROTOTYPES = {
     "ginn_hip_sync": (c_int, [c_void_p]),
     "ginn_hip_malloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "ginn_hip_free": (c_int, [c_void_p, c_void_p]),
+    "ginn_hip_pool_configure": (c_int, [c_void_p, c_int, c_size_t]),
+    "ginn_hip_pool_trim": (c_int, [c_void_p]),
+    "ginn_hip_pool_stats": (c_int, [c_void_p, POINTER(c_size_t), POINTER(c_size_t)]),
     "ginn_hip_memcpy_h2d": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "ginn_hip_memcpy_d2h": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "ginn_hip_memcpy_d2d": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),

@@ -9,6 +9,8 @@
 #include <cstdint>
 #include <cstdio>
 #include <mutex>
+#include <unordered_map>
+#include <vector>
 
 #include "../../include/ginn_hip.h"
 
@@ -50,6 +52,18 @@ void clear_error();
 // Context
 // ---------------------------------------------------------------------------
 
+// Free device blocks kept for reuse, by block size.  Every block is used on the
+// context's one stream only, so a block released by the host may be handed out
+// again at once: whatever still reads it was enqueued earlier on that stream.
+struct ginn_hip_pool {
+  std::mutex mutex;
+  std::unordered_map<size_t, std::vector<void*>> free_blocks;  // block size -> blocks
+  std::unordered_map<void*, size_t> block_size;                // every live or cached block of the pool
+  size_t cached_bytes = 0;
+  size_t limit_bytes = size_t(8) << 30;  // beyond this, released blocks go back to the driver
+  bool enabled = true;
+};
+
 struct ginn_hip_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
@@ -65,6 +79,7 @@ struct ginn_hip_ctx {
   std::mutex mutex;  // serialises workspace users across host threads
   hipEvent_t events[64] = {};
   int num_cus = 256;
+  ginn_hip_pool pool;
 };
 
 // A recorded sequence of launches on a context's stream.

@@ -120,6 +120,27 @@ int stage_to_workspace(ginn_hip_ctx* ctx, size_t offset, const void* host_src,
 
 }  // namespace ginn_hip
 
+namespace {
+// Block sizes of the pool: powers of two from 256 B to 2 MiB, multiples of 2 MiB above.
+size_t pool_block_size(size_t bytes) {
+  constexpr size_t kLarge = size_t(2) << 20;
+  if (bytes > kLarge) return (bytes + kLarge - 1) / kLarge * kLarge;
+  size_t b = 256;
+  while (b < bytes) b <<= 1;
+  return b;
+}
+// Gives every cached block back to the driver; the caller holds the pool's mutex.
+void pool_release_cached(ginn_hip_pool& pool) {
+  for (auto& [size, blocks] : pool.free_blocks)
+    for (void* p : blocks) {
+      (void)hipFree(p);
+      pool.block_size.erase(p);
+    }
+  pool.free_blocks.clear();
+  pool.cached_bytes = 0;
+}
+}  // namespace
+
 using namespace ginn_hip;
 
 extern "C" {
@@ -161,6 +182,7 @@ int ginn_hip_ctx_destroy(ginn_hip_ctx* ctx) {
   if (ctx->staging_event) (void)hipEventDestroy(ctx->staging_event);
   if (ctx->host_staging) (void)hipHostFree(ctx->host_staging);
   if (ctx->workspace) (void)hipFree(ctx->workspace);
+  pool_release_cached(ctx->pool);
   if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
   return kOk;
@@ -189,12 +211,32 @@ int ginn_hip_malloc(ginn_hip_ctx* ctx, size_t bytes, void** ptr) {
   *ptr = nullptr;
   if (bytes == 0) return kOk;
   GH_HIP(hipSetDevice(ctx->device));
-  hipError_t e = hipMalloc(ptr, bytes);
+  ginn_hip_pool& pool = ctx->pool;
+  std::lock_guard<std::mutex> lock(pool.mutex);
+  const size_t block = pool.enabled ? pool_block_size(bytes) : bytes;
+  if (pool.enabled) {
+    auto it = pool.free_blocks.find(block);
+    if (it != pool.free_blocks.end() && !it->second.empty()) {
+      *ptr = it->second.back();
+      it->second.pop_back();
+      pool.cached_bytes -= block;
+      return kOk;
+    }
+  }
+  hipError_t e = hipMalloc(ptr, block);
+  if (e == hipErrorOutOfMemory && pool.cached_bytes > 0) {
+    // The cache holds what the driver lacks: give it back and ask again.
+    (void)hipGetLastError();
+    pool_release_cached(pool);
+    e = hipMalloc(ptr, block);
+  }
   if (e != hipSuccess) {
     (void)hipGetLastError();
+    *ptr = nullptr;
     return fail(e == hipErrorOutOfMemory ? kOutOfMemory : kHipError,
                 "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
   }
+  if (pool.enabled) pool.block_size[*ptr] = block;
   return kOk;
 }
 
@@ -202,7 +244,50 @@ int ginn_hip_free(ginn_hip_ctx* ctx, void* ptr) {
   GH_CHECK_ARG(ctx, "ginn_hip_free: ctx is NULL");
   if (!ptr) return kOk;
   GH_HIP(hipSetDevice(ctx->device));
+  ginn_hip_pool& pool = ctx->pool;
+  std::lock_guard<std::mutex> lock(pool.mutex);
+  auto it = pool.block_size.find(ptr);
+  if (it != pool.block_size.end()) {
+    const size_t block = it->second;
+    if (pool.enabled && pool.cached_bytes + block <= pool.limit_bytes) {
+      pool.free_blocks[block].push_back(ptr);
+      pool.cached_bytes += block;
+      return kOk;
+    }
+    pool.block_size.erase(it);
+  }
   GH_HIP(hipFree(ptr));
+  return kOk;
+}
+
+int ginn_hip_pool_configure(ginn_hip_ctx* ctx, int enabled, size_t limit_bytes) {
+  GH_CHECK_ARG(ctx, "ginn_hip_pool_configure: ctx is NULL");
+  GH_HIP(hipSetDevice(ctx->device));
+  ginn_hip_pool& pool = ctx->pool;
+  std::lock_guard<std::mutex> lock(pool.mutex);
+  pool.enabled = enabled != 0;
+  pool.limit_bytes = limit_bytes;
+  if (!pool.enabled || pool.cached_bytes > pool.limit_bytes) {
+    GH_HIP(hipStreamSynchronize(ctx->stream));
+    pool_release_cached(pool);
+  }
+  return kOk;
+}
+
+int ginn_hip_pool_trim(ginn_hip_ctx* ctx) {
+  GH_CHECK_ARG(ctx, "ginn_hip_pool_trim: ctx is NULL");
+  GH_HIP(hipSetDevice(ctx->device));
+  GH_HIP(hipStreamSynchronize(ctx->stream));
+  std::lock_guard<std::mutex> lock(ctx->pool.mutex);
+  pool_release_cached(ctx->pool);
+  return kOk;
+}
+
+int ginn_hip_pool_stats(ginn_hip_ctx* ctx, size_t* cached_bytes, size_t* blocks) {
+  GH_CHECK_ARG(ctx && cached_bytes && blocks, "ginn_hip_pool_stats: NULL argument");
+  std::lock_guard<std::mutex> lock(ctx->pool.mutex);
+  *cached_bytes = ctx->pool.cached_bytes;
+  *blocks = ctx->pool.block_size.size();
   return kOk;
 }
 

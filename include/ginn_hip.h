@@ -107,9 +107,22 @@ int ginn_hip_sync(ginn_hip_ctx* ctx);
 /* Memory  (ginn/dev.h:158-175, 269-343)                               */
 /* ------------------------------------------------------------------ */
 
-/* GpuDevice::alloc / ::free (ginn/dev.h:158-175). */
+/* GpuDevice::alloc / ::free (ginn/dev.h:158-175).  Where the reference calls
+ * cudaMalloc / cudaFree per temporary tensor, released blocks are kept by the
+ * context (sizes rounded to powers of two up to 2 MiB, to multiples of 2 MiB
+ * above) and handed out again without a driver call.  That is safe because a
+ * context's memory is only used on its one stream: whatever still reads a
+ * released block was enqueued before the block's next user.  Memory obtained
+ * here must not be used on another stream without the caller's own ordering. */
 int ginn_hip_malloc(ginn_hip_ctx* ctx, size_t bytes, void** ptr);
 int ginn_hip_free(ginn_hip_ctx* ctx, void* ptr);
+/* The cache of released blocks: switch it off (enabled = 0: malloc / free go to
+ * the driver as in the reference), bound it (default 8 GiB; blocks released
+ * beyond the bound go back to the driver), empty it (waits for the stream), or
+ * read it (bytes held for reuse, and blocks the pool knows, in use or held). */
+int ginn_hip_pool_configure(ginn_hip_ctx* ctx, int enabled, size_t limit_bytes);
+int ginn_hip_pool_trim(ginn_hip_ctx* ctx);
+int ginn_hip_pool_stats(ginn_hip_ctx* ctx, size_t* cached_bytes, size_t* blocks);
 
 /* Device::copy, GPU<-CPU branch: asynchronous on the stream
  * (ginn/dev.h:276-280).  `host_src` must stay valid until the stream reaches
