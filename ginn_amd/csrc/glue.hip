@@ -284,7 +284,7 @@ __global__ __launch_bounds__(kBlock) void pick_nls_bwd_kernel(int rows, int cols
                                                               const typename T::storage* __restrict__ smax,
                                                               const int* __restrict__ idx,
                                                               const typename T::storage* __restrict__ dout,
-                                                              typename T::storage* dx) {
+                                                              typename T::storage* dx, int accumulate) {
   const size_t n = static_cast<size_t>(rows) * cols;
   GH_GRID_STRIDE_V(i, n, V) {
     const int r = static_cast<int>(i % rows);
@@ -292,7 +292,12 @@ __global__ __launch_bounds__(kBlock) void pick_nls_bwd_kernel(int rows, int cols
     const float g = to_float<T>(dout[c]);
     const int hot = idx[c] - r;  // position of the picked row inside this vector, if any
     float v[V], sm[V];
-    ld<T, V>(dx + i, v);
+    if (accumulate) {
+      ld<T, V>(dx + i, v);
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[e] = 0.f;
+    }
     ld<T, V>(smax + i, sm);
 #pragma unroll
     for (int e = 0; e < V; ++e) v[e] += sm[e] * g - (e == hot ? g : 0.f);
@@ -481,20 +486,31 @@ int ginn_hip_pick_nls_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int
   return kOk;
 }
 
-int ginn_hip_pick_nls_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* smax,
-                          const int* idx, const void* dout, void* dx) {
-  GH_CHECK_ARG(ctx, "ginn_hip_pick_nls_bwd: ctx is NULL");
-  GH_CHECK_ARG(rows >= 1 && cols >= 0, "ginn_hip_pick_nls_bwd: bad dimension");
+static int pick_nls_bwd(const char* who, ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols,
+                        const void* smax, const int* idx, const void* dout, void* dx, int accumulate) {
+  GH_CHECK_ARG(ctx, "%s: ctx is NULL", who);
+  GH_CHECK_ARG(rows >= 1 && cols >= 0, "%s: bad dimension", who);
   if (cols == 0) return kOk;
-  GH_CHECK_ARG(smax && idx && dout && dx, "ginn_hip_pick_nls_bwd: NULL pointer");
+  GH_CHECK_ARG(smax && idx && dout && dx, "%s: NULL pointer", who);
   GH_HIP(hipSetDevice(ctx->device));
   const bool vec = vec8_ok({smax, dx}, {static_cast<size_t>(rows)});
   const size_t total = static_cast<size_t>(rows) * cols;
   const unsigned grid = grid_for(vec ? total / 8 : total, kBlock, ctx->num_cus);
   GH_DISPATCH_DTYPE_V(dtype, vec, (pick_nls_bwd_kernel<T, V><<<grid, kBlock, 0, ctx->stream>>>(
-      rows, cols, static_cast<const T::storage*>(smax), idx, static_cast<const T::storage*>(dout), static_cast<T::storage*>(dx))));
+      rows, cols, static_cast<const T::storage*>(smax), idx, static_cast<const T::storage*>(dout), static_cast<T::storage*>(dx),
+      accumulate)));
   GH_HIP(hipGetLastError());
   return kOk;
+}
+
+int ginn_hip_pick_nls_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* smax,
+                          const int* idx, const void* dout, void* dx) {
+  return pick_nls_bwd("ginn_hip_pick_nls_bwd", ctx, dtype, rows, cols, smax, idx, dout, dx, 1);
+}
+
+int ginn_hip_pick_nls_bwd_assign(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* smax,
+                                 const int* idx, const void* dout, void* dx) {
+  return pick_nls_bwd("ginn_hip_pick_nls_bwd_assign", ctx, dtype, rows, cols, smax, idx, dout, dx, 0);
 }
 
 }  // extern "C"

@@ -140,8 +140,20 @@ double run_passes(LevelExecutor& ex, int iters) {
 // of consecutive levels joined into chain launches.
 int g_exec_mode = 0;
 
+// Zero fills made on demand during the timed passes of the last run_warm(): a
+// gradient that reset_grad() had only flagged was read or added to before its
+// user overwrote it.  None are expected; each is a launch of its own.
+long g_timed_fills = 0;
+
+struct FillCount {
+  size_t before = internal::lazy_grad_settles();
+  void start() { before = internal::lazy_grad_settles(); }
+  ~FillCount() { g_timed_fills = static_cast<long>(internal::lazy_grad_settles() - before); }
+};
+
 // Warm-up pass (first-touch allocations, launch plans), then `iters` timed ones.
 double run_warm(Graph& g, int iters) {
+  FillCount count;
   if (g_exec_mode & 2) {
     LevelExecutor ex(g);
     run_passes(ex, 1);
@@ -150,11 +162,14 @@ double run_warm(Graph& g, int iters) {
     if ((g_exec_mode & 12) == 12) {
       ex.record_pass();
       ex.replay_pass();  // the first replay also loads the graph onto the device
+      count.start();
       return run_replays(ex, iters);
     }
+    count.start();
     return run_passes(ex, iters);
   }
   run_passes(g, 1);
+  count.start();
   return run_passes(g, iters);
 }
 
@@ -375,12 +390,15 @@ int lstm(int mode, int nseq, const int* lens, int E, int H, const float* W, cons
     if ((mode & 12) == 12) {       // ... as one recorded device graph
       ex.record_pass();
       ex.replay_pass();
+      FillCount count;
       ms = run_replays(ex, iters);
     } else {
+      FillCount count;
       ms = run_passes(ex, iters);
     }
   } else {
     first_ms = run_passes(g, 1);
+    FillCount count;
     ms = run_passes(g, iters);
     if (out_launches) *out_launches = 0;
   }
@@ -479,6 +497,9 @@ int gpt_layer(int C, int nh, int B, int T, int V, const float* x, const int* tar
 extern "C" {
 
 const char* scenario_last_error() { return g_error.c_str(); }
+
+// Zero fills on demand during the timed passes of the last scenario (see g_timed_fills).
+long scenario_timed_fills() { return g_timed_fills; }
 
 int scenario_mlp(int dtype, int batch, int n_layers, const int* dims, const int* acts, const float* x,
                  const int* labels, const float* const* W, const float* const* b, int iters, float* out_loss,

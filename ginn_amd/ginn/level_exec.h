@@ -98,6 +98,16 @@ class LevelExecutor {
   };
   std::vector<Step> steps_[3];
   std::vector<LaunchDesc> descs_;  // scratch of the pass under way (keeps its capacity)
+  // Nodes whose gradient reset_grad() flags instead of zeroing (BaseNode::GradUse),
+  // as of the last pass that was not frozen.
+  std::vector<BaseNode*> lazy_;
+  // Those of them whose flag a node takes while it runs itself: only these
+  // are flagged again in frozen passes (a recorded launch asks nothing).
+  std::vector<BaseNode*> lazy_direct_;
+  std::vector<BaseNode*> taken_by_plans_;
+  // A flagged gradient was zeroed on demand while a node described its work:
+  // that fill is in no plan, so the passes cannot be replayed from plans.
+  bool unplanned_fill_ = false;
   bool frozen_ = false;
   ginn_hip_graph* pass_graph_ = nullptr;  // a recorded frozen pass (record_pass())
 
@@ -611,6 +621,9 @@ class LevelExecutor {
   // reset_grad() and backward() must have run once before.
   LevelExecutor& freeze() {
     for (auto& steps : steps_) GINN_ASSERT(!steps.empty(), "LevelExecutor::freeze() before a full pass");
+    GINN_ASSERT(!unplanned_fill_,
+                "LevelExecutor::freeze(): a node that declares GradUse::Overwrites added to a gradient that "
+                "reset_grad() had only flagged; run with set_lazy_grad_reset(false)");
     frozen_ = true;
     return *this;
   }
@@ -712,10 +725,12 @@ class LevelExecutor {
 
   LevelExecutor& reset_grad() {
     if (frozen_ && fused_ready_) {
+      for (BaseNode* n : lazy_direct_) n->reset_grad_lazy();
       run_fused(kReset);
       return *this;
     }
     if (frozen_) {
+      for (BaseNode* n : lazy_direct_) n->reset_grad_lazy();
       for (Step& step : steps_[kReset]) {
         for (BaseNode* n : step.direct) n->reset_grad();
         if (step.plan >= 0) launch(plans_[kReset][static_cast<size_t>(step.plan)]);
@@ -724,11 +739,17 @@ class LevelExecutor {
     }
     cursor_ = 0;
     descs_.clear();
+    lazy_.clear();
+    const std::vector<unsigned char> lazy = lazy_grad_candidates(list_);
     Step& step = begin_step(kReset, 0);
-    for (auto& n : list_) {  // graph order: views map onto gradients sized before them
-      if (!n->describe_reset_grad(descs_)) {
+    for (size_t i = 0; i < list_.size(); ++i) {  // graph order: views map onto gradients sized before them
+      BaseNode* n = list_[i].get();
+      if (lazy[i]) {
+        n->reset_grad_lazy();
+        lazy_.push_back(n);
+      } else if (!n->describe_reset_grad(descs_)) {
         n->reset_grad();
-        step.direct.push_back(n.get());
+        step.direct.push_back(n);
       }
     }
     flush(kReset, step);
@@ -739,30 +760,46 @@ class LevelExecutor {
   // level; reset_grad() must have run (ginn/node.h:237-254).
   LevelExecutor& backward(double loss_coeff = 1) {
     seed_sink(loss_coeff);
-    if (frozen_ && fused_ready_) {
-      run_fused(kBackward);
-      return *this;
-    }
     if (frozen_) {
-      for (Step& step : steps_[kBackward]) {
-        for (BaseNode* n : step.direct) n->backward();
-        if (step.plan >= 0) launch(plans_[kBackward][static_cast<size_t>(step.plan)]);
+      if (fused_ready_) {
+        run_fused(kBackward);
+      } else {
+        for (Step& step : steps_[kBackward]) {
+          for (BaseNode* n : step.direct) n->backward();
+          if (step.plan >= 0) launch(plans_[kBackward][static_cast<size_t>(step.plan)]);
+        }
       }
+      for (BaseNode* n : lazy_direct_) n->clear_lazy_zero();  // all taken already, unless a node returned early
       return *this;
     }
     cursor_ = 0;
     descs_.clear();
+    unplanned_fill_ = false;
+    taken_by_plans_.clear();
+    struct LogGuard {
+      ~LogGuard() { internal::lazy_take_log() = nullptr; }
+    } guard;
     for (size_t k = 0; k < levels_.size(); ++k) {
       Step& step = begin_step(kBackward, k);
       for (BaseNode* n : levels_[levels_.size() - 1 - k]) {
         if (!n->has_grad()) continue;
-        if (!n->describe_backward(descs_)) {
+        const size_t fills = internal::lazy_grad_settles();
+        internal::lazy_take_log() = &taken_by_plans_;
+        const bool described = n->describe_backward(descs_);
+        internal::lazy_take_log() = nullptr;
+        if (!described) {
           n->backward();
           step.direct.push_back(n);
+        } else if (internal::lazy_grad_settles() != fills) {
+          unplanned_fill_ = true;
         }
       }
       flush(kBackward, step);
     }
+    std::sort(taken_by_plans_.begin(), taken_by_plans_.end());
+    lazy_direct_.clear();
+    for (BaseNode* n : lazy_)
+      if (!std::binary_search(taken_by_plans_.begin(), taken_by_plans_.end(), n)) lazy_direct_.push_back(n);
     return *this;
   }
 

@@ -190,6 +190,35 @@ class BaseNode {
   virtual bool has_grad() const { return false; }
   virtual void init_grad() {}
   virtual void reset_grad() {}
+
+  // ---- gradients that are cleared lazily -----------------------------------
+  // A gradient with exactly one writer that can overwrite need not be zeroed
+  // and then added to: Graph::reset_grad() (and the level executor's) only
+  // flags such a gradient as "holds no value yet", and the writer, which asks
+  // with take_lazy_zero() before it touches the gradient, then overwrites it
+  // (a product runs with beta = 0).  Everything else sees zeros: reading a
+  // flagged gradient through grad() clears it first.  The reference zeroes
+  // every gradient in reset_grad() (ginn/node.h:218-222) and adds in every
+  // backward; the values are the same, one write and one read of each such
+  // gradient are not made.
+  enum class GradUse {
+    Accumulates,  // backward adds to the input's gradient (every node may)
+    Overwrites,   // backward asks take_lazy_zero() of the input first and overwrites when told to
+    Aliases       // this node's gradient IS the whole of the input's (views, in-place nodes)
+  };
+  // How backward() treats the gradient of input `index`.
+  virtual GradUse grad_use(size_t /*index*/) const { return GradUse::Accumulates; }
+  // The node holds gradient storage of its own that may be flagged.
+  virtual bool owns_grad() const { return false; }
+  // reset_grad() that may flag instead of zeroing.
+  virtual void reset_grad_lazy() { reset_grad(); }
+  // True exactly once after a lazy reset: the caller must now overwrite the
+  // whole gradient.  Views and in-place nodes ask their input.
+  virtual bool take_lazy_zero() { return false; }
+  virtual bool lazy_zero() const { return false; }
+  // Drops the flag without clearing: for an executor whose recorded launches
+  // have overwritten the gradient.
+  virtual void clear_lazy_zero() {}
   virtual void reset_forwarded() { forwarded = false; }
   virtual std::string name() const = 0;
 };
@@ -216,6 +245,9 @@ class Node : public BaseNode {
   virtual const Tensor<Scalar>& grad() const = 0;
   Tensor<Scalar>& value() { return const_cast<Tensor<Scalar>&>(std::as_const(*this).value()); }
   Tensor<Scalar>& grad() { return const_cast<Tensor<Scalar>&>(std::as_const(*this).grad()); }
+
+  // The gradient tensor as it is, flagged or not: for views that map onto it.
+  virtual Tensor<Scalar>& grad_storage() { return grad(); }
 
   DevPtr dev() const override { return value().dev(); }
   Shape shape() const override { return value().shape(); }
@@ -263,6 +295,65 @@ template <typename Scalar = Real>
 using NodePtr = Ptr<Node<Scalar>>;
 template <typename Scalar = Real>
 using ConstNodePtr = Ptr<const Node<Scalar>>;
+
+namespace internal {
+inline bool& lazy_grad_reset_flag() {
+  static bool on = true;
+  return on;
+}
+// Zero fills made on demand because a flagged gradient was read or added to
+// before anything overwrote it (process-wide, for tests and the executor).
+inline std::atomic<size_t>& lazy_grad_settles() {
+  static std::atomic<size_t> n{0};
+  return n;
+}
+// While set, every gradient whose flag is taken is noted here (the level
+// executor tells apart the flags that recorded launches consume).
+inline std::vector<BaseNode*>*& lazy_take_log() {
+  thread_local std::vector<BaseNode*>* log = nullptr;
+  return log;
+}
+}  // namespace internal
+
+// Whether reset_grad() of Graph and LevelExecutor may flag gradients instead of
+// zeroing them (BaseNode::GradUse); on by default.
+inline void set_lazy_grad_reset(bool on) { internal::lazy_grad_reset_flag() = on; }
+inline bool lazy_grad_reset() { return internal::lazy_grad_reset_flag(); }
+
+// For a node list in graph order (inputs first): out[i] != 0 iff the gradient
+// of list[i] may be flagged instead of zeroed.  That takes storage of its own,
+// exactly one use as an input within the list, and a user that overwrites --
+// directly, or through a chain of views and in-place nodes each with one use.
+inline std::vector<unsigned char> lazy_grad_candidates(const std::vector<BaseNodePtr>& list) {
+  const size_t n = list.size();
+  std::vector<unsigned char> out(n, 0);
+  if (!internal::lazy_grad_reset_flag()) return out;
+  const uint64_t epoch = BaseNode::new_epoch();
+  for (size_t i = 0; i < n; ++i) list[i]->mark(epoch, i);
+  std::vector<uint32_t> uses(n, 0), user(n, 0), slot(n, 0);
+  for (size_t u = 0; u < n; ++u) {
+    const auto& ins = list[u]->inputs();
+    for (size_t k = 0; k < ins.size(); ++k) {
+      if (!ins[k]->marked(epoch)) continue;
+      const size_t j = ins[k]->mark_value();
+      ++uses[j];
+      user[j] = static_cast<uint32_t>(u);
+      slot[j] = static_cast<uint32_t>(k);
+    }
+  }
+  std::vector<unsigned char> overwritten(n, 0);  // by the one user, were the gradient flagged
+  for (size_t j = n; j-- > 0;) {                 // users come later in the list
+    BaseNode& node = *list[j];
+    if (uses[j] != 1 || !node.has_grad()) continue;
+    BaseNode& u = *list[user[j]];
+    if (!u.has_grad()) continue;
+    const BaseNode::GradUse use = u.grad_use(slot[j]);
+    if (use == BaseNode::GradUse::Overwrites) overwritten[j] = 1;
+    else if (use == BaseNode::GradUse::Aliases) overwritten[j] = overwritten[user[j]];
+    out[j] = overwritten[j] && node.owns_grad();
+  }
+  return out;
+}
 
 class Graph {
   std::vector<BaseNodePtr> list_;
@@ -327,8 +418,14 @@ class Graph {
     for (auto& e : list_) e->init_grad();
     return *this;
   }
+  // Gradients with a single overwriting user are flagged, not zeroed
+  // (BaseNode::GradUse); all others are zeroed as in ginn/node.h:218-222.
   Graph& reset_grad() {
-    for (auto& e : list_) e->reset_grad();
+    const std::vector<unsigned char> lazy = lazy_grad_candidates(list_);
+    for (size_t i = 0; i < list_.size(); ++i) {
+      if (lazy[i]) list_[i]->reset_grad_lazy();
+      else list_[i]->reset_grad();
+    }
     return *this;
   }
   Graph& reset_forwarded() {

@@ -73,8 +73,14 @@ class AffineNode : public BaseDataNode<Scalar> {
                                           bias->has_grad() ? bias->grad().data() : nullptr));
     for (size_t i = 0; i + 1 < ins_.size(); i += 2) {
       auto &a = ins_[i], &b = ins_[i + 1];
-      if (b->has_grad()) gpu_prod(b->grad(), a->value(), daffine, ProdResult::Add, ProdTranspose::First);
-      if (a->has_grad()) gpu_prod(a->grad(), daffine, b->value(), ProdResult::Add, ProdTranspose::Second);
+      if (b->has_grad()) {
+        const bool fresh = b->take_lazy_zero();
+        gpu_prod(b->grad(), a->value(), daffine, fresh ? ProdResult::Assign : ProdResult::Add, ProdTranspose::First);
+      }
+      if (a->has_grad()) {
+        const bool fresh = a->take_lazy_zero();
+        gpu_prod(a->grad(), daffine, b->value(), fresh ? ProdResult::Assign : ProdResult::Add, ProdTranspose::Second);
+      }
     }
   }
 
@@ -113,6 +119,10 @@ class AffineNode : public BaseDataNode<Scalar> {
       : AffineNode(nonlin, std::vector<NodePtr<Scalar>>({in, args...})) {}
 
   const NonlinOp<Scalar>& nonlin() const { return *nonlin_; }
+  // Products overwrite; the bias gradient is added to.
+  BaseNode::GradUse grad_use(size_t index) const override {
+    return index + 1 < ins_.size() ? BaseNode::GradUse::Overwrites : BaseNode::GradUse::Accumulates;
+  }
   std::string name() const override { return "AffineNode"; }
 };
 

@@ -44,13 +44,17 @@ class AddNode : public BaseDataNode<Scalar> {
     internal::add_tensors(value(), srcs, false);
   }
   void backward_() override {
-    for (auto& in : ins_)
-      if (in->has_grad()) internal::add_tensors(in->grad(), {&grad()}, true);
+    for (auto& in : ins_) {
+      if (!in->has_grad()) continue;
+      const bool fresh = in->take_lazy_zero();
+      internal::add_tensors(in->grad(), {&grad()}, !fresh);
+    }
   }
 
  public:
   using BaseDataNode<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
+  BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; }
 
   bool describe_forward(std::vector<LaunchDesc>& out) override {
     if (value().dev()->kind() != GPU) return false;
@@ -77,7 +81,7 @@ class AddNode : public BaseDataNode<Scalar> {
       LaunchDesc d;
       d.dtype = dtype_of<Scalar>();
       d.kind = GINN_HIP_MULTI_SUM;
-      d.accumulate = true;
+      d.accumulate = !in->take_lazy_zero();
       d.n = static_cast<size_t>(grad().size());
       d.dst = in->grad().data();
       d.src[0] = grad().data();
@@ -115,13 +119,20 @@ class CwiseProdNode : public BaseDataNode<Scalar> {
     run(value(), a_->value(), b_->value(), false);
   }
   void backward_() override {
-    if (a_->has_grad()) run(a_->grad(), grad(), b_->value(), true);
-    if (b_->has_grad()) run(b_->grad(), grad(), a_->value(), true);
+    if (a_->has_grad()) {
+      const bool fresh = a_->take_lazy_zero();
+      run(a_->grad(), grad(), b_->value(), !fresh);
+    }
+    if (b_->has_grad()) {
+      const bool fresh = b_->take_lazy_zero();
+      run(b_->grad(), grad(), a_->value(), !fresh);
+    }
   }
 
  public:
   using BaseDataNode<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
+  BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; }
   LaunchDesc prod_desc(Scalar* dst, const Scalar* x, const Scalar* y, bool accumulate) const {
     LaunchDesc d;
     d.dtype = dtype_of<Scalar>();
@@ -142,8 +153,14 @@ class CwiseProdNode : public BaseDataNode<Scalar> {
   }
   bool describe_backward(std::vector<LaunchDesc>& out) override {
     if (value().dev()->kind() != GPU) return false;
-    if (a_->has_grad()) out.push_back(prod_desc(a_->grad().data(), grad().data(), b_->value().data(), true));
-    if (b_->has_grad()) out.push_back(prod_desc(b_->grad().data(), grad().data(), a_->value().data(), true));
+    if (a_->has_grad()) {
+      const bool fresh = a_->take_lazy_zero();
+      out.push_back(prod_desc(a_->grad().data(), grad().data(), b_->value().data(), !fresh));
+    }
+    if (b_->has_grad()) {
+      const bool fresh = b_->take_lazy_zero();
+      out.push_back(prod_desc(b_->grad().data(), grad().data(), a_->value().data(), !fresh));
+    }
     return true;
   }
   CwiseProdNode(const NodePtr<Scalar>& a, const NodePtr<Scalar>& b) : BaseDataNode<Scalar>({a, b}), a_(a), b_(b) {}
@@ -174,15 +191,17 @@ class ScaleShiftNode : public BaseDataNode<Scalar> {
                                        value().data(), 0));
   }
   void backward_() override {
-    if (in_->has_grad())
-      GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(grad()), dtype_of<Scalar>(),
-                                         static_cast<size_t>(grad().size()), alpha_, 0.f, grad().data(),
-                                         in_->grad().data(), 1));
+    if (!in_->has_grad()) return;
+    const bool fresh = in_->take_lazy_zero();
+    GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(grad()), dtype_of<Scalar>(),
+                                       static_cast<size_t>(grad().size()), alpha_, 0.f, grad().data(),
+                                       in_->grad().data(), fresh ? 0 : 1));
   }
 
  public:
   using BaseDataNode<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
+  BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; }
   ScaleShiftNode(const NodePtr<Scalar>& in, float alpha, float shift, const char* name)
       : BaseDataNode<Scalar>({in}), in_(in), alpha_(alpha), shift_(shift), name_(name) {}
   std::string name() const override { return name_; }

@@ -12,6 +12,7 @@ template <typename Scalar = Real>
 class BaseDataNode : public Node<Scalar> {
   Tensor<Scalar> fx_, dfx_;
   bool has_grad_ = true;
+  mutable bool lazy_zero_ = false;  // dfx_ holds no value yet: see BaseNode::GradUse
 
  public:
   BaseDataNode(DevPtr dev, const std::vector<BaseNodePtr>& ins) : Node<Scalar>(ins), fx_(dev), dfx_(dev) {}
@@ -29,15 +30,74 @@ class BaseDataNode : public Node<Scalar> {
       : BaseDataNode(dev, std::vector<BaseNodePtr>(ins)) {}
 
   const Tensor<Scalar>& value() const override { return fx_; }
-  const Tensor<Scalar>& grad() const override { return dfx_; }
+  // A gradient flagged by reset_grad_lazy() is cleared before anybody sees it.
+  const Tensor<Scalar>& grad() const override {
+    if (lazy_zero_) {
+      lazy_zero_ = false;
+      const_cast<Tensor<Scalar>&>(dfx_).set_zero();
+      ++internal::lazy_grad_settles();
+    }
+    return dfx_;
+  }
   using Node<Scalar>::value;
   using Node<Scalar>::grad;
+  Tensor<Scalar>& grad_storage() override { return dfx_; }
+
+  bool owns_grad() const override { return is_floating_point_v<Scalar>; }
+  void reset_grad_lazy() override {
+    if (!this->owns_grad()) {  // a view or an in-place node built on this class
+      this->reset_grad();
+      return;
+    }
+    lazy_zero_ = false;
+    this->init_grad();
+    lazy_zero_ = this->has_grad() && dfx_.size() > 0;
+  }
+  bool take_lazy_zero() override {
+    const bool was = lazy_zero_;
+    lazy_zero_ = false;
+    if (was && internal::lazy_take_log()) internal::lazy_take_log()->push_back(this);
+    return was;
+  }
+  bool lazy_zero() const override { return lazy_zero_; }
+  void clear_lazy_zero() override { lazy_zero_ = false; }
 
   bool has_grad() const override { return has_grad_; }
   virtual void set_has_grad(bool hg) { has_grad_ = hg; }
 
   std::string name() const override = 0;
 };
+
+// Inside a node whose gradient tensor is a view of the WHOLE gradient of the
+// node IN (its input 0): the flag of a lazily reset gradient lives in IN.
+#define GINN_GRAD_IS_VIEW_OF(IN)                                                               \
+  bool owns_grad() const override { return false; }                                            \
+  bool take_lazy_zero() override { return IN->take_lazy_zero(); }                              \
+  bool lazy_zero() const override { return IN->lazy_zero(); }                                  \
+  void clear_lazy_zero() override {}                                                           \
+  BaseNode::GradUse grad_use(size_t index) const override {                                    \
+    return index == 0 ? BaseNode::GradUse::Aliases : BaseNode::GradUse::Accumulates;           \
+  }                                                                                            \
+  const Tensor<Scalar>& grad() const override {                                                \
+    if (IN->lazy_zero()) (void)std::as_const(*IN).grad();                                      \
+    return BaseDataNode<Scalar>::grad();                                                       \
+  }                                                                                            \
+  using Node<Scalar>::grad;
+
+// Inside a node whose grad() IS the gradient tensor of the node IN (its input 0):
+// IN sizes and clears it, this node has nothing to prepare.
+#define GINN_GRAD_IS_ALIAS_OF(IN)                                                              \
+  void init_grad() override {}                                                                 \
+  void reset_grad() override {}                                                                \
+  bool describe_reset_grad(std::vector<LaunchDesc>&) override { return true; }                 \
+  bool owns_grad() const override { return false; }                                            \
+  bool take_lazy_zero() override { return IN->take_lazy_zero(); }                              \
+  bool lazy_zero() const override { return IN->lazy_zero(); }                                  \
+  void clear_lazy_zero() override {}                                                           \
+  Tensor<Scalar>& grad_storage() override { return IN->grad_storage(); }                       \
+  BaseNode::GradUse grad_use(size_t index) const override {                                    \
+    return index == 0 ? BaseNode::GradUse::Aliases : BaseNode::GradUse::Accumulates;           \
+  }
 
 // A node whose value is a row of column blocks, one per part: where each part
 // starts and how many columns it has, as of the last forward pass.  What

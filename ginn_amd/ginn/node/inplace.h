@@ -36,6 +36,7 @@ class InPlaceProdScalarNode : public BaseDataNode<Scalar> {
   using Node<Scalar>::value;
   using Node<Scalar>::grad;
   bool has_grad() const override { return in_->has_grad(); }
+  GINN_GRAD_IS_ALIAS_OF(in_)
   template <typename Val>
   InPlaceProdScalarNode(const NodePtr<Scalar>& in, Val val)
       : BaseDataNode<Scalar>({in}), in_(in), val_(static_cast<float>(val)) {}
@@ -76,6 +77,7 @@ class InPlaceMaskNode : public BaseDataNode<Scalar> {
   using Node<Scalar>::value;
   using Node<Scalar>::grad;
   bool has_grad() const override { return in_->has_grad(); }
+  GINN_GRAD_IS_ALIAS_OF(in_)
   template <typename Val>
   InPlaceMaskNode(const NodePtr<Scalar>& in, const NodePtr<Scalar>& mask, Val mask_val)
       : BaseDataNode<Scalar>({in, mask}), in_(in), mask_(mask), mask_val_(static_cast<float>(mask_val)) {}
@@ -91,6 +93,7 @@ GINN_MAKE_SCALAR_FORWARDING_FACTORY(InPlaceMask);
   using Node<Scalar>::value;                                                                   \
   using Node<Scalar>::grad;                                                                    \
   bool has_grad() const override { return IN->has_grad(); }                                    \
+  GINN_GRAD_IS_ALIAS_OF(IN)                                                                    \
   bool describe_forward(std::vector<LaunchDesc>&) override { return false; }                   \
   bool describe_backward(std::vector<LaunchDesc>&) override { return false; }
 
@@ -235,6 +238,7 @@ class InPlacePermuteNode : public PermuteNode<Scalar> {
     this->overwrite_ = true;
   }
   bool has_grad() const override { return in_->has_grad(); }
+  bool owns_grad() const override { return false; }  // the input's gradient under the permuted shape
   void init_grad() override {
     if (this->has_grad()) this->grad().map(in_->grad(), PermuteNode<Scalar>::permute(in_->shape(), indices_));
   }

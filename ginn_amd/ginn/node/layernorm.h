@@ -28,14 +28,16 @@ class LayerNormNode : public BaseDataNode<Scalar> {
   void backward_() override {
     if (!in_->has_grad()) return;
     auto& y = value();
-    GINN_HIP_CALL(ginn_hip_layernorm_bwd(internal::ctx_of(y), dtype_of<Scalar>(), static_cast<int>(y.rows()),
-                                         static_cast<int>(y.cols()), grad().data(), y.data(), std_.data(),
-                                         in_->grad().data()));
+    const bool fresh = in_->take_lazy_zero();
+    GINN_HIP_CALL((fresh ? ginn_hip_layernorm_bwd_assign : ginn_hip_layernorm_bwd)(
+        internal::ctx_of(y), dtype_of<Scalar>(), static_cast<int>(y.rows()), static_cast<int>(y.cols()),
+        grad().data(), y.data(), std_.data(), in_->grad().data()));
   }
 
  public:
   using BaseDataNode<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
+  BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; }
   LayerNormNode(const NodePtr<Scalar>& in, double eps = 1e-8)
       : BaseDataNode<Scalar>({in}), in_(in), eps_(static_cast<float>(eps)), std_(in->dev()) {}
   std::string name() const override { return "LayerNorm"; }

@@ -228,6 +228,7 @@ class RowwiseUncatNode : public BaseDataNode<Scalar> {
   using BaseDataNode<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
   bool has_grad() const override { return in_->has_grad(); }
+  bool owns_grad() const override { return false; }  // a window of x's gradient
   void init_grad() override {
     if (!has_grad()) return;
     const Size off = cat_->offsets().at(static_cast<size_t>(index_));
@@ -294,6 +295,7 @@ class ColBroadcastNode : public BaseDataNode<Scalar> {
     if (cols_->value() == 1) return in_->has_grad();
     return BaseDataNode<Scalar>::has_grad();
   }
+  bool owns_grad() const override { return false; }  // with one column the gradient is the input's
   void init_grad() override {
     if (!has_grad()) return;
     if (cols_->value() > 1) {
@@ -406,10 +408,10 @@ class ReshapeNode : public BaseDataNode<Scalar> {
 
  public:
   using BaseDataNode<Scalar>::value;
-  using BaseDataNode<Scalar>::grad;
+  GINN_GRAD_IS_VIEW_OF(in_)
   bool has_grad() const override { return in_->has_grad(); }
   void init_grad() override {
-    if (has_grad()) grad().map(in_->grad(), shape_);
+    if (has_grad()) this->grad_storage().map(in_->grad_storage(), shape_);
   }
   void reset_grad() override { init_grad(); }
   // A view has nothing to launch: mapping is all of its work in every pass.
@@ -436,10 +438,10 @@ class MapNode : public BaseDataNode<Scalar> {
 
  public:
   using BaseDataNode<Scalar>::value;
-  using BaseDataNode<Scalar>::grad;
+  GINN_GRAD_IS_VIEW_OF(in_)
   bool has_grad() const override { return in_->has_grad(); }
   void init_grad() override {
-    if (has_grad()) grad().map(in_->grad());
+    if (has_grad()) this->grad_storage().map(in_->grad_storage());
   }
   void reset_grad() override { init_grad(); }
   // A view has nothing to launch: mapping is all of its work in every pass.
@@ -514,13 +516,17 @@ class PermuteNode : public BaseDataNode<Scalar> {
       flat.map(in_->grad(), in_->shape());
       flat = tmp;
     } else {
-      run(grad(), grad().shape(), inverse(indices_), in_->grad(), true);
+      const bool fresh = in_->take_lazy_zero();
+      run(grad(), grad().shape(), inverse(indices_), in_->grad(), !fresh);
     }
   }
 
  public:
   using BaseDataNode<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
+  BaseNode::GradUse grad_use(size_t) const override {
+    return overwrite_ ? BaseNode::GradUse::Accumulates : BaseNode::GradUse::Overwrites;
+  }
   PermuteNode(const NodePtr<Scalar>& in, Shape indices)
       : BaseDataNode<Scalar>({in}), in_(in), indices_(std::move(indices)) {}
   std::string name() const override { return "Permute"; }

@@ -15,13 +15,16 @@ namespace ginn {
     F##Op<Scalar> op_{};                                                       \
     void forward_() override { op_.forward(value(), in_->value()); }           \
     void backward_() override {                                                \
-      if (in_->has_grad()) op_.backward(in_->grad(), grad(), in_->value(), value(), true); \
+      if (!in_->has_grad()) return;                                            \
+      const bool fresh = in_->take_lazy_zero();                                \
+      op_.backward(in_->grad(), grad(), in_->value(), value(), !fresh);        \
     }                                                                          \
                                                                                \
    public:                                                                     \
     using BaseDataNode<Scalar>::value;                                         \
     using BaseDataNode<Scalar>::grad;                                          \
     using UnaryOp = F##Op<Scalar>;                                             \
+    BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; } \
     bool describe_forward(std::vector<LaunchDesc>& out) override {             \
       if (value().dev()->kind() != GPU || op_.code() == GINN_HIP_ACT_SOFTMAX) return false; \
       value().resize(in_->value().shape());                                    \
@@ -42,7 +45,7 @@ namespace ginn {
       d.dtype = dtype_of<Scalar>();                                            \
       d.kind = GINN_HIP_MULTI_NONLIN_BWD;                                      \
       d.act = op_.code();                                                      \
-      d.accumulate = true;                                                     \
+      d.accumulate = !in_->take_lazy_zero();                                   \
       d.n = static_cast<size_t>(value().size());                               \
       d.dst = in_->grad().data();                                              \
       d.src[0] = grad().data();                                                \
@@ -90,6 +93,7 @@ GINN_MAKE_UNARY_NODE_AND_FACTORY(Gelu2);
     using Node<Scalar>::value;                                                 \
     using Node<Scalar>::grad;                                                  \
     bool has_grad() const override { return in_->has_grad(); }                 \
+    GINN_GRAD_IS_ALIAS_OF(in_)                                                 \
     bool describe_forward(std::vector<LaunchDesc>&) override { return false; } \
     bool describe_backward(std::vector<LaunchDesc>&) override { return false; } \
     using UnaryOp = F##Op<Scalar>;                                             \

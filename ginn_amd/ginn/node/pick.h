@@ -113,15 +113,19 @@ class PickNegLogSoftmaxNode : public PickSoftmaxNode<Scalar> {
   void backward_() override {
     if (!in_->has_grad()) return;
     auto& x = in_->value();
-    GINN_HIP_CALL(ginn_hip_pick_nls_bwd(internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()),
-                                        static_cast<int>(x.cols()), smax_.data(), index_->value().data(),
-                                        grad().data(), in_->grad().data()));
+    const bool fresh = in_->take_lazy_zero();
+    GINN_HIP_CALL((fresh ? ginn_hip_pick_nls_bwd_assign : ginn_hip_pick_nls_bwd)(
+        internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()), static_cast<int>(x.cols()),
+        smax_.data(), index_->value().data(), grad().data(), in_->grad().data()));
   }
 
  public:
   using BaseDataNode<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
   using PickSoftmaxNode<Scalar>::PickSoftmaxNode;
+  BaseNode::GradUse grad_use(size_t index) const override {
+    return index == 0 ? BaseNode::GradUse::Overwrites : BaseNode::GradUse::Accumulates;
+  }
   std::string name() const override { return "PickNegLogSoftmax"; }
 };
 GINN_MAKE_SCALAR_FORWARDING_FACTORY(PickNegLogSoftmax);

@@ -23,8 +23,14 @@ class ProdNode : public BaseDataNode<Scalar> {
   }
   void backward_() override {
     using namespace internal;
-    if (b_->has_grad()) gpu_prod(b_->grad(), a_->value(), grad(), ProdResult::Add, ProdTranspose::First);
-    if (a_->has_grad()) gpu_prod(a_->grad(), grad(), b_->value(), ProdResult::Add, ProdTranspose::Second);
+    if (b_->has_grad()) {
+      const bool fresh = b_->take_lazy_zero();
+      gpu_prod(b_->grad(), a_->value(), grad(), fresh ? ProdResult::Assign : ProdResult::Add, ProdTranspose::First);
+    }
+    if (a_->has_grad()) {
+      const bool fresh = a_->take_lazy_zero();
+      gpu_prod(a_->grad(), grad(), b_->value(), fresh ? ProdResult::Assign : ProdResult::Add, ProdTranspose::Second);
+    }
   }
 
  public:
@@ -33,6 +39,7 @@ class ProdNode : public BaseDataNode<Scalar> {
   using BaseDataNode<Scalar>::grad;
 
   ProdNode(const NodePtr<Scalar>& a, const NodePtr<Scalar>& b) : BaseDataNode<Scalar>({a, b}), a_(a), b_(b) {}
+  BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; }
 
   void set_ins(const std::vector<BaseNodePtr>& ins) override {
     GINN_ASSERT(ins.size() == 2);
@@ -150,10 +157,11 @@ class GatherProdNode : public BaseDataNode<Scalar>, public ColumnPartition {
       // dA[m x k] += dY[m x total] * X^T, X's columns gathered: they are the
       // stored columns of the transposed operand, indexed along the sum.
       auto* table = static_cast<const void* const*>(values_.commit(dev(), ctx));
+      const bool fresh = a_->take_lazy_zero();
       GINN_HIP_CALL(ginn_hip_gemm_gathered(ctx, dtype_of<Scalar>(), internal::OP_N, internal::OP_T,
                                            static_cast<int>(m), static_cast<int>(k), static_cast<int>(total),
-                                           grad().data(), static_cast<int>(m), nullptr, 0, table, 1.f,
-                                           a_->grad().data(), static_cast<int>(m), nullptr,
+                                           grad().data(), static_cast<int>(m), nullptr, 0, table,
+                                           fresh ? 0.f : 1.f, a_->grad().data(), static_cast<int>(m), nullptr,
                                            values_.aligned()));
     }
     size_t with_grad = 0;
@@ -207,6 +215,11 @@ class GatherProdNode : public BaseDataNode<Scalar>, public ColumnPartition {
 
   const std::vector<Size>& offsets() const override { return offsets_; }
   const std::vector<Size>& extents() const override { return extents_; }
+  // The left operand's gradient may be overwritten; the gathered ones are added
+  // to by one launch for all of them, which has one beta.
+  BaseNode::GradUse grad_use(size_t index) const override {
+    return index == 0 ? BaseNode::GradUse::Overwrites : BaseNode::GradUse::Accumulates;
+  }
 
   void set_ins(const std::vector<BaseNodePtr>& ins) override {
     GINN_ASSERT(ins.size() >= 2);
@@ -240,10 +253,16 @@ class BatchedProdNode : public BaseDataNode<Scalar> {
   }
   void backward_() override {
     using namespace internal;
-    if (a_->has_grad())
-      gpu_batched_prod(a_->grad(), grad(), b_->value(), ProdResult::Add, ProdTranspose::Second);
-    if (b_->has_grad())
-      gpu_batched_prod(b_->grad(), a_->value(), grad(), ProdResult::Add, ProdTranspose::First);
+    if (a_->has_grad()) {
+      const bool fresh = a_->take_lazy_zero();
+      gpu_batched_prod(a_->grad(), grad(), b_->value(), fresh ? ProdResult::Assign : ProdResult::Add,
+                       ProdTranspose::Second);
+    }
+    if (b_->has_grad()) {
+      const bool fresh = b_->take_lazy_zero();
+      gpu_batched_prod(b_->grad(), a_->value(), grad(), fresh ? ProdResult::Assign : ProdResult::Add,
+                       ProdTranspose::First);
+    }
   }
 
  public:
@@ -253,6 +272,7 @@ class BatchedProdNode : public BaseDataNode<Scalar> {
 
   BatchedProdNode(const NodePtr<Scalar>& a, const NodePtr<Scalar>& b)
       : BaseDataNode<Scalar>({a, b}), a_(a), b_(b) {}
+  BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; }
   std::string name() const override { return "BatchedProd"; }
 };
 

@@ -24,6 +24,7 @@ class WeightNode : public Node<Scalar> {
   std::shared_ptr<Tensor<Scalar>> fx_;
   std::shared_ptr<std::mutex> access_;
   bool has_grad_ = true;
+  mutable bool lazy_zero_ = false;  // dfx_ holds no value yet: see BaseNode::GradUse
 
  public:
   std::string label;
@@ -52,8 +53,31 @@ class WeightNode : public Node<Scalar> {
     GINN_ASSERT(static_cast<bool>(fx_));
     return *fx_;
   }
-  const Tensor<Scalar>& grad() const override { return dfx_; }
+  // A gradient flagged by reset_grad_lazy() is cleared before anybody sees it.
+  const Tensor<Scalar>& grad() const override {
+    if (lazy_zero_) {
+      lazy_zero_ = false;
+      const_cast<Tensor<Scalar>&>(dfx_).set_zero();
+      ++internal::lazy_grad_settles();
+    }
+    return dfx_;
+  }
   using Node<Scalar>::grad;
+  Tensor<Scalar>& grad_storage() override { return dfx_; }
+  bool owns_grad() const override { return is_floating_point_v<Scalar>; }
+  void reset_grad_lazy() override {
+    lazy_zero_ = false;
+    this->init_grad();
+    lazy_zero_ = owns_grad() && has_grad_ && dfx_.size() > 0;
+  }
+  bool take_lazy_zero() override {
+    const bool was = lazy_zero_;
+    lazy_zero_ = false;
+    if (was && internal::lazy_take_log()) internal::lazy_take_log()->push_back(this);
+    return was;
+  }
+  bool lazy_zero() const override { return lazy_zero_; }
+  void clear_lazy_zero() override { lazy_zero_ = false; }
 
   bool has_grad() const override { return has_grad_; }
   virtual void set_has_grad(bool hg) { has_grad_ = hg; }

@@ -363,6 +363,12 @@ int ginn_hip_pick_nls_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows,
 int ginn_hip_pick_nls_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows,
                           int cols, const void* smax, const int* idx,
                           const void* dout, void* dx);
+/* The same with `=` in place of `+=`: what the backward pass of
+ * ginn/node/pick.h:226-236 leaves in a gradient that reset_grad() had just
+ * zeroed (ginn/node.h:218-222), without reading the zeros. */
+int ginn_hip_pick_nls_bwd_assign(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                                 int rows, int cols, const void* smax,
+                                 const int* idx, const void* dout, void* dx);
 
 /* ------------------------------------------------------------------ */
 /* Transformer-block companions (column-major, fp32 statistics)        */

@@ -55,7 +55,9 @@ def test_one_launch_per_level(phases):
 
 def test_reset_is_one_zero_fill(phases):
     calls, _, direct = phases["reset 1"]
-    assert len(calls) == 1 and calls[0][0] == "multi_zero" and calls[0][1] >= 10
+    # one fill for every gradient that is zeroed; those with a single overwriting
+    # user are only flagged (BaseNode::GradUse) and are in no launch
+    assert len(calls) == 1 and calls[0][0] == "multi_zero" and calls[0][1] >= 5
     assert direct == 0
 
 

@@ -1,0 +1,119 @@
+"""Gradients that reset_grad() flags instead of zeroing (BaseNode::GradUse in
+ginn_amd/ginn/node.h).  The reference zeroes every gradient in reset_grad()
+(ginn/node.h:218-222) and adds in every backward pass; a gradient with one
+user that can overwrite is only flagged here and the user overwrites it (a
+product runs with beta = 0).  The gradients must not depend on that: one graph
+with every overwriting node as a sole user (attention block, gated product,
+vocabulary head; tests/cpp/lazy_shim.cpp) is run with the flagging on and off,
+node by node and through the level executor in every mode, over several passes."""
+import ctypes
+import math
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+from conftest import rel_fro
+from ginn_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+SHIM = Path(__file__).resolve().parent / "cpp" / "libhost_shim.so"
+MODES = {"graph": 0, "executor": 1, "frozen": 2, "chained": 3, "recorded": 4}
+
+
+@pytest.fixture(scope="module")
+def shim():
+    if not SHIM.exists():
+        pytest.fail(f"{SHIM} is missing: run __graft_entry__.build()")
+    capi.load()
+    lib = ctypes.CDLL(str(SHIM))
+    lib.lazy_last_error.restype = ctypes.c_char_p
+    return lib
+
+
+def fptr(a):
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+
+
+def run(lib, dt, lazy, mode, passes, hs=16, nh=2, B=3, T=24, V=40, seed=0):
+    from gpu_util import round_to
+    C = hs * nh
+    rng = np.random.default_rng(seed)
+    shapes = [(C, C), (C,), (C, C), (C,), (C, C), (C,), (C, C), (C, C), (V, C), (V,)]
+    params = [np.asfortranarray(round_to(rng.uniform(-1, 1, s) / math.sqrt(C), dt).astype(np.float32)) for s in shapes]
+    x = np.asfortranarray(round_to(rng.uniform(-1, 1, (C, B, T)), dt).astype(np.float32))
+    targets = rng.integers(0, V, B * T).astype(np.int32)
+    grads = [np.zeros(s, np.float32, order="F") for s in shapes]
+    dx = np.zeros((C, B, T), np.float32, order="F")
+    loss = np.zeros(1, np.float32)
+    flagged = ctypes.c_long(-1)
+    fills = ctypes.c_long(-1)
+    pp = (ctypes.POINTER(ctypes.c_float) * 10)(*[fptr(p) for p in params])
+    gp = (ctypes.POINTER(ctypes.c_float) * 10)(*[fptr(g) for g in grads])
+    rc = lib.shim_lazy_graph(dt, lazy, MODES[mode], passes, hs, nh, B, T, V, fptr(x),
+                             targets.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), pp, fptr(loss), fptr(dx), gp,
+                             ctypes.byref(flagged), ctypes.byref(fills))
+    assert rc == 0, lib.lazy_last_error().decode()
+    return loss[0], dx, grads, flagged.value, fills.value
+
+
+@pytest.mark.parametrize("dt", [capi.F32, capi.F16, capi.BF16])
+@pytest.mark.parametrize("mode", list(MODES))
+def test_flagged_gradients_equal_zeroed_ones(shim, dt, mode):
+    """Same loss and gradients with and without the flagging, after three passes
+    (a stale flag or a gradient that was neither zeroed nor overwritten would
+    show as last pass's gradient added in, or as zeros)."""
+    want_loss, want_dx, want_grads, none, _ = run(shim, dt, 0, "graph", 1)
+    assert none == 0
+    got_loss, got_dx, got_grads, flagged, fills = run(shim, dt, 1, mode, 3)
+    # 19 float nodes of the graph have a single user that overwrites (directly or
+    # through views and in-place nodes); none of them needed a fill on demand.
+    assert flagged >= 15, flagged
+    assert fills == 0, fills
+    # beta = 0 instead of 0 + 1 * x changes no rounding; the split of a long sum
+    # over workgroups may differ between the two launches of a product.
+    # 16-bit storage: the executor adds the users of one gradient in another order than the node-by-node
+    # pass does, which moves a result by one unit of the last place (2^-11 for f16, 2^-8 for bf16).
+    tol = {capi.F32: 1e-6, capi.F16: 2e-3, capi.BF16: 1e-2}[dt]
+    assert abs(got_loss - want_loss) <= tol * max(1.0, abs(want_loss))
+    assert np.abs(want_dx).max() > 0
+    assert rel_fro(got_dx, want_dx) <= tol
+    for g, w in zip(got_grads, want_grads):
+        assert np.abs(w).max() > 0
+        assert rel_fro(g, w) <= tol
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+def test_switch_off_matches_in_every_mode(shim, mode):
+    """set_lazy_grad_reset(false): nothing is flagged and every mode still
+    agrees with the node-by-node pass."""
+    want_loss, want_dx, want_grads, _, _ = run(shim, capi.F32, 0, "graph", 1, seed=3)
+    got_loss, got_dx, got_grads, flagged, fills = run(shim, capi.F32, 0, mode, 2, seed=3)
+    assert flagged == 0 and fills == 0
+    assert rel_fro(got_dx, want_dx) <= 1e-6
+    for g, w in zip(got_grads, want_grads):
+        assert rel_fro(g, w) <= 1e-6
+
+
+def test_reading_a_flagged_gradient_gives_zeros(shim):
+    out = np.full(1, -1, np.float32)
+    assert shim.shim_lazy_semantics(0, fptr(out)) == 0, shim.lazy_last_error().decode()
+    assert out[0] == 0.0
+
+
+def test_graphs_that_share_a_node(shim):
+    """Two graphs over one product node, reset one after the other, run one after
+    the other: the first user overwrites, the second adds (ginn/node.h:237-254
+    accumulates over both)."""
+    out = np.zeros(1, np.float32)
+    assert shim.shim_lazy_semantics(1, fptr(out)) == 0, shim.lazy_last_error().decode()
+    assert out[0] == pytest.approx(1 - math.tanh(4.0) ** 2 + 3.0, rel=1e-6)
+
+
+def test_only_single_overwriting_users_qualify(shim):
+    out = np.zeros(1, np.float32)
+    assert shim.shim_lazy_semantics(2, fptr(out)) == 0, shim.lazy_last_error().decode()
+    # A, B (Prod overwrites), Sum(P) and Sum(Q) (Add overwrites); not P (three
+    # uses), not Q (Sum adds to its input), not the sink.
+    assert out[0] == 4

@@ -25,6 +25,7 @@ def shim():
     capi.load()
     lib = ctypes.CDLL(str(SHIM))
     lib.scenario_last_error.restype = ctypes.c_char_p
+    lib.scenario_timed_fills.restype = ctypes.c_long
     return lib
 
 
@@ -305,8 +306,10 @@ def test_lstm_level_executor_full_config(shim, gather):
     assert stats["launches"] < stats["nodes"] / 10
     got, want, stats = run_lstm(shim, 7, lens, 128, 256, seed=9, iters=3)
     compare_lstm(got, want)
+    assert shim.scenario_timed_fills() == 0  # no gradient was zeroed on demand, one launch each
     fused, want, fstats = run_lstm(shim, 23, lens, 128, 256, seed=9, iters=3)
     compare_lstm(fused, want)
+    assert shim.scenario_timed_fills() == 0
     for key in ("h", "dxs", "db", "dW"):
         np.testing.assert_array_equal(fused[key], got[key], err_msg=key)
     assert fstats["launches"] < stats["launches"] / 2

@@ -192,6 +192,9 @@ def run_gpt(shim, dt, C, nh, B, T, V, seed, iters=1, wscale=0.02):
         (FP * 20)(*[a.ctypes.data_as(FP) for a in grads]), dx.ctypes.data_as(FP), ctypes.byref(ms),
         ctypes.byref(nodes))
     assert rc == 0, shim.scenario_last_error().decode()
+    # no gradient that reset_grad() had only flagged was read or added to before its user overwrote it
+    shim.scenario_timed_fills.restype = ctypes.c_long
+    assert shim.scenario_timed_fills() == 0
     p64 = N.GptBlockParams(**{k: np.asfortranarray(v.astype(np.float64)) for k, v in params.items()})
     wloss, wgrads = N.gpt_layer_forward_backward(p64, np.asfortranarray(x.astype(np.float64)), targets, nh)
     got = dict(zip(N.GptBlockParams.NAMES, grads))
