@@ -68,6 +68,23 @@ class BaseDataNode : public Node<Scalar> {
   std::string name() const override = 0;
 };
 
+// An in-place step (scale, mask) that postpones its work until somebody reads
+// its value: a Softmax directly after it then does scale, mask and softmax as
+// one launch over the scores (ginn_hip_scaled_masked_softmax_fwd) instead of
+// three.  Whoever else reads the value first triggers the step as usual.
+class PendingInPlace {
+ public:
+  enum class Step { Scale, Mask };
+  virtual ~PendingInPlace() = default;
+  virtual Step pending_step() const = 0;
+  virtual bool pending() const = 0;
+  virtual void take_pending() = 0;             // the caller does the step itself
+  virtual float pending_value() const = 0;     // the factor, or the value for masked entries
+  virtual BaseNode* pending_mask() const { return nullptr; }
+  virtual BaseNode* pending_input() const = 0;  // the node whose storage the step writes over
+  virtual void skip_next_backward() = 0;        // the caller has done this step's backward too
+};
+
 // Inside a node whose gradient tensor is a view of the WHOLE gradient of the
 // node IN (its input 0): the flag of a lazily reset gradient lives in IN.
 #define GINN_GRAD_IS_VIEW_OF(IN)                                                               \

@@ -16,26 +16,49 @@ namespace ginn {
 // x *= val in place; the gradient is scaled in place on the way back
 // (ginn/node/inplace.h:104-123).
 template <typename Scalar>
-class InPlaceProdScalarNode : public BaseDataNode<Scalar> {
+class InPlaceProdScalarNode : public BaseDataNode<Scalar>, public PendingInPlace {
   NodePtr<Scalar> in_;
   float val_;
+  mutable bool pending_ = false;  // forward() has run, the scaling has not (PendingInPlace)
+  bool skip_backward_ = false;
 
-  void scale(Tensor<Scalar>& t) {
+  void scale(Tensor<Scalar>& t) const {
     internal::require_gpu(t.dev(), "InPlaceProdScalar");
     GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(t), dtype_of<Scalar>(), static_cast<size_t>(t.size()), val_,
                                        0.f, t.data(), t.data(), 0));
   }
-  void forward_() override { scale(in_->value()); }
+  void forward_() override {
+    internal::require_gpu(in_->dev(), "InPlaceProdScalar");
+    pending_ = true;
+  }
   void backward_() override {
+    if (skip_backward_) {
+      skip_backward_ = false;
+      return;
+    }
     if (in_->has_grad()) scale(in_->grad());
   }
 
  public:
-  const Tensor<Scalar>& value() const override { return std::as_const(*in_).value(); }
+  const Tensor<Scalar>& value() const override {
+    if (pending_) {
+      pending_ = false;
+      scale(in_->value());
+    }
+    return std::as_const(*in_).value();
+  }
   const Tensor<Scalar>& grad() const override { return std::as_const(*in_).grad(); }
   using Node<Scalar>::value;
   using Node<Scalar>::grad;
+  Shape shape() const override { return in_->shape(); }
+  DevPtr dev() const override { return in_->dev(); }
   bool has_grad() const override { return in_->has_grad(); }
+  Step pending_step() const override { return Step::Scale; }
+  bool pending() const override { return pending_; }
+  void take_pending() override { pending_ = false; }
+  float pending_value() const override { return val_; }
+  BaseNode* pending_input() const override { return in_.get(); }
+  void skip_next_backward() override { skip_backward_ = true; }
   GINN_GRAD_IS_ALIAS_OF(in_)
   template <typename Val>
   InPlaceProdScalarNode(const NodePtr<Scalar>& in, Val val)
@@ -48,35 +71,57 @@ GINN_MAKE_SCALAR_FORWARDING_FACTORY(InPlaceProdScalar);
 // over the trailing dimensions in which it has extent 1.  Backward zeroes the
 // gradient at the masked entries (ginn/node/inplace.h:152-212).
 template <typename Scalar>
-class InPlaceMaskNode : public BaseDataNode<Scalar> {
+class InPlaceMaskNode : public BaseDataNode<Scalar>, public PendingInPlace {
   NodePtr<Scalar> in_, mask_;
   float mask_val_;
+  mutable bool pending_ = false;  // forward() has run, the masking has not (PendingInPlace)
+  bool skip_backward_ = false;
 
-  void fill(Tensor<Scalar>& t, float v) {
+  void fill(Tensor<Scalar>& t, float v) const {
     internal::require_gpu(t.dev(), "InPlaceMask");
     const Size ms = mask_->value().size();
     GINN_HIP_CALL(ginn_hip_mask_fill(internal::ctx_of(t), dtype_of<Scalar>(), static_cast<size_t>(ms),
                                      static_cast<size_t>(t.size() / ms), mask_->value().data(), v, t.data()));
   }
   void forward_() override {
-    const Shape ms = mask_->value().shape(), is = in_->value().shape();
+    const Shape ms = mask_->value().shape(), is = in_->shape();  // shape(), not value(): a pending step below stays so
     GINN_ASSERT(ms.size() == is.size(), "InPlaceMask: mask and input ranks differ");
     size_t i = 0;
     while (i < is.size() && ms[i] == is[i]) ++i;
     for (; i < is.size(); ++i) GINN_ASSERT(ms[i] == 1, "Unexpected mask shape!");
     GINN_ASSERT(mask_->value().size() > 0);
-    fill(in_->value(), mask_val_);
+    internal::require_gpu(in_->dev(), "InPlaceMask");
+    pending_ = true;
   }
   void backward_() override {
+    if (skip_backward_) {
+      skip_backward_ = false;
+      return;
+    }
     if (in_->has_grad()) fill(in_->grad(), 0.f);
   }
 
  public:
-  const Tensor<Scalar>& value() const override { return std::as_const(*in_).value(); }
+  const Tensor<Scalar>& value() const override {
+    if (pending_) {
+      pending_ = false;
+      fill(in_->value(), mask_val_);  // in_->value() first runs a step pending below
+    }
+    return std::as_const(*in_).value();
+  }
   const Tensor<Scalar>& grad() const override { return std::as_const(*in_).grad(); }
   using Node<Scalar>::value;
   using Node<Scalar>::grad;
+  Shape shape() const override { return in_->shape(); }
+  DevPtr dev() const override { return in_->dev(); }
   bool has_grad() const override { return in_->has_grad(); }
+  Step pending_step() const override { return Step::Mask; }
+  bool pending() const override { return pending_; }
+  void take_pending() override { pending_ = false; }
+  float pending_value() const override { return mask_val_; }
+  BaseNode* pending_mask() const override { return mask_.get(); }
+  BaseNode* pending_input() const override { return in_.get(); }
+  void skip_next_backward() override { skip_backward_ = true; }
   GINN_GRAD_IS_ALIAS_OF(in_)
   template <typename Val>
   InPlaceMaskNode(const NodePtr<Scalar>& in, const NodePtr<Scalar>& mask, Val mask_val)

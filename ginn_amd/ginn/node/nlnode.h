@@ -68,7 +68,95 @@ GINN_MAKE_UNARY_NODE_AND_FACTORY(Identity);
 GINN_MAKE_UNARY_NODE_AND_FACTORY(Tanh);
 GINN_MAKE_UNARY_NODE_AND_FACTORY(Sigmoid);
 GINN_MAKE_UNARY_NODE_AND_FACTORY(Relu);
-GINN_MAKE_UNARY_NODE_AND_FACTORY(Softmax);
+
+// Softmax down the columns.  Directly after InPlaceMask (and InPlaceProdScalar
+// before that) whose work is still pending -- the score chain of an attention
+// block, examples/min-gpt.cu.cpp:127-133 -- the three steps run as one launch,
+// forward and, when the scores' gradient holds no value yet, backward; the
+// results are those of the separate nodes, bit for bit.
+template <typename Scalar>
+using ColumnSoftmaxOp = SoftmaxOp<Scalar>;
+GINN_MAKE_UNARY_NODE_AND_FACTORY(ColumnSoftmax);
+
+template <typename Scalar>
+class SoftmaxNode : public ColumnSoftmaxNode<Scalar> {
+  using Base = ColumnSoftmaxNode<Scalar>;
+  using Base::in_;
+
+  struct Chain {
+    PendingInPlace* mask_step = nullptr;
+    PendingInPlace* scale_step = nullptr;  // may be absent
+    Node<Scalar>* mask = nullptr;
+    Node<Scalar>* scores = nullptr;  // the node whose storage the steps write over
+  };
+  // The in-place steps directly before this node, if they are a mask step with
+  // an optional scale step below.
+  Chain chain() const {
+    Chain c;
+    auto* m = dynamic_cast<PendingInPlace*>(in_.get());
+    if (!m || m->pending_step() != PendingInPlace::Step::Mask) return c;
+    auto* mask = dynamic_cast<Node<Scalar>*>(m->pending_mask());
+    BaseNode* below = m->pending_input();
+    auto* p = dynamic_cast<PendingInPlace*>(below);
+    if (p && p->pending_step() == PendingInPlace::Step::Scale) {
+      c.scale_step = p;
+      below = p->pending_input();
+    }
+    auto* scores = dynamic_cast<Node<Scalar>*>(below);
+    if (!mask || !scores) return Chain{};
+    c.mask_step = m;
+    c.mask = mask;
+    c.scores = scores;
+    return c;
+  }
+
+  void forward_() override {
+    const Chain c = chain();
+    // Pending below means: nobody has read the scaled / masked scores yet.  A
+    // scale step that has run already (somebody read its value) counts as 1.
+    if (!c.mask_step || !c.mask_step->pending() || in_->dev()->kind() != GPU) {
+      Base::forward_();
+      return;
+    }
+    float scale = 1.f;
+    if (c.scale_step && c.scale_step->pending()) {
+      scale = c.scale_step->pending_value();
+      c.scale_step->take_pending();
+    }
+    c.mask_step->take_pending();
+    Tensor<Scalar>& x = c.scores->value();
+    this->value().resize(x.shape());
+    GINN_HIP_CALL(ginn_hip_scaled_masked_softmax_fwd(
+        internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()), static_cast<int>(x.cols()), x.data(),
+        scale, c.mask->value().data(), static_cast<size_t>(c.mask->value().size()), c.mask_step->pending_value(),
+        this->value().data()));
+  }
+
+  void backward_() override {
+    if (!in_->has_grad()) return;
+    const Chain c = chain();
+    // A flagged gradient below means: this node is the only user of the mask
+    // step, that of the scale step, and so on down to the scores (BaseNode::GradUse).
+    if (!c.mask_step || !in_->lazy_zero() || in_->dev()->kind() != GPU) {
+      Base::backward_();
+      return;
+    }
+    in_->take_lazy_zero();
+    const Tensor<Scalar>& y = this->value();
+    GINN_HIP_CALL(ginn_hip_scaled_masked_softmax_bwd(
+        internal::ctx_of(y), dtype_of<Scalar>(), static_cast<int>(y.rows()), static_cast<int>(y.cols()),
+        this->grad().data(), y.data(), c.scale_step ? c.scale_step->pending_value() : 1.f, c.mask->value().data(),
+        static_cast<size_t>(c.mask->value().size()), in_->grad().data()));
+    c.mask_step->skip_next_backward();
+    if (c.scale_step) c.scale_step->skip_next_backward();
+  }
+
+ public:
+  using Base::Base;
+  using UnaryOp = SoftmaxOp<Scalar>;
+  std::string name() const override { return "Softmax"; }
+};
+GINN_MAKE_SCALAR_FORWARDING_FACTORY(Softmax);
 GINN_MAKE_UNARY_NODE_AND_FACTORY(Log);
 GINN_MAKE_UNARY_NODE_AND_FACTORY(Sqrt);
 GINN_MAKE_UNARY_NODE_AND_FACTORY(Gelu);

@@ -417,6 +417,27 @@ int ginn_hip_mask_fill(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
                        size_t mask_size, size_t batch, const void* mask,
                        float value, void* x);
 
+/* The score chain of an attention block as one pass: InPlaceProdScalar
+ * (ginn/node/inplace.h:104-123), InPlaceMask (:152-212) and Softmax
+ * (ginn/nonlin.h:162-168) over x [rows x cols], softmax down the columns.
+ *   x <- scale * x;  x[i] <- fill where mask[i % mask_n] == 0;  y = softmax(x)
+ * x is updated in place, as the two in-place nodes leave it; y is a different
+ * array.  mask has the operand's dtype and mask_n divides rows * cols.  Every
+ * step rounds to the storage type like the separate calls (ginn_hip_scale_shift,
+ * ginn_hip_mask_fill, ginn_hip_nonlin_fwd) do: same bits, one read of x. */
+int ginn_hip_scaled_masked_softmax_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                                       int rows, int cols, void* x, float scale,
+                                       const void* mask, size_t mask_n,
+                                       float fill, void* y);
+/* The three backward steps (ginn/nonlin.h:170-188, ginn/node/inplace.h:198-212
+ * and :118-122) for a gradient that holds no value yet:
+ *   dx = scale * (mask ? y (*) (dy - colsum(y (*) dy)) : 0), assigned. */
+int ginn_hip_scaled_masked_softmax_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                                       int rows, int cols, const void* dy,
+                                       const void* y, float scale,
+                                       const void* mask, size_t mask_n,
+                                       void* dx);
+
 /* UpperTriNode (ginn/node/layout.h:922-955): dst [n x n] = 1 where
  * row <= col, else 0. */
 int ginn_hip_upper_tri(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int n,

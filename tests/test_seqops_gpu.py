@@ -168,6 +168,107 @@ def test_upper_tri_and_mask_fill(dev, dt, n, batch):
 
 
 # ---------------------------------------------------------------------------
+# scale -> mask -> softmax of attention scores as one launch
+# ---------------------------------------------------------------------------
+
+# (T, batch, offset): scores [T x T x batch], causal mask [T x T]; an offset breaks 16-byte alignment.
+# 512: one vector per lane, two columns per wave; 1024, 2048: 2 and 4 vectors; 24: a partly filled
+# wave; 20 (rows % 8 != 0), 4096 (column too long for the registers) and the offset case take the
+# three separate launches inside the entry point.
+SCORE_CASES = [(512, 3, 0), (1024, 1, 0), (2048, 1, 0), (24, 5, 0), (64, 7, 0), (20, 3, 0), (24, 2, 1)]
+
+
+def _score_inputs(dev, dt, T, batch, offset, seed):
+    from gpu_util import round_to
+    rng = np.random.default_rng(seed)
+    x = round_to(rng.standard_normal((T, T * batch)) * 3, dt)
+    dy = round_to(rng.standard_normal((T, T * batch)), dt)
+    mask = N.upper_tri(T).astype(np.float32)
+    return x, dy, mask
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("T,batch,offset", SCORE_CASES + [(4096, 1, 0)])
+def test_scaled_masked_softmax_equals_the_three_steps(dev, dt, T, batch, offset):
+    """ginn_hip_scaled_masked_softmax_fwd / _bwd against ginn_hip_scale_shift, ginn_hip_mask_fill and
+    ginn_hip_nonlin_fwd / _bwd called one after the other (what InPlaceProdScalar, InPlaceMask and
+    Softmax do as three nodes): the same bits, in the scores left in place, the softmax and the gradient
+    (the gradient in half storage: up to the last bit of a few results per million, see below)."""
+    if T == 4096 and dt != capi.BF16:
+        pytest.skip("one dtype is enough for the long-column fallback")
+    x, dy, mask = _score_inputs(dev, dt, T, batch, offset, seed=T + batch)
+    n = x.size
+    scale = 1.0 / np.sqrt(64.0)
+    flat = lambda a: a.reshape(-1, order="F")
+    bm, pm, _ = dev.put(flat(mask), dt)
+    # separate steps
+    bx1, px1, _ = dev.put(flat(x), dt, offset=offset)
+    by1, py1, _ = dev.put(np.zeros(n), dt, offset=offset)
+    dev.lib.call("ginn_hip_scale_shift", dev.ctx, dt, n, scale, 0.0, c_void_p(px1), c_void_p(px1), 0)
+    dev.lib.call("ginn_hip_mask_fill", dev.ctx, dt, T * T, batch, c_void_p(pm), float("-inf"), c_void_p(px1))
+    dev.lib.call("ginn_hip_nonlin_fwd", dev.ctx, dt, capi.ACT_SOFTMAX, T, T * batch, c_void_p(px1), c_void_p(py1))
+    bg, pg, _ = dev.put(flat(dy), dt, offset=offset)
+    bd1, pd1, _ = dev.put(np.full(n, 7.0), dt, offset=offset)  # overwritten: accumulate = 0
+    dev.lib.call("ginn_hip_nonlin_bwd", dev.ctx, dt, capi.ACT_SOFTMAX, T, T * batch, c_void_p(pg), None,
+                 c_void_p(py1), c_void_p(pd1), 0)
+    dev.lib.call("ginn_hip_mask_fill", dev.ctx, dt, T * T, batch, c_void_p(pm), 0.0, c_void_p(pd1))
+    dev.lib.call("ginn_hip_scale_shift", dev.ctx, dt, n, scale, 0.0, c_void_p(pd1), c_void_p(pd1), 0)
+    # one launch each way
+    bx2, px2, _ = dev.put(flat(x), dt, offset=offset)
+    by2, py2, _ = dev.put(np.zeros(n), dt, offset=offset)
+    dev.lib.call("ginn_hip_scaled_masked_softmax_fwd", dev.ctx, dt, T, T * batch, c_void_p(px2), scale, c_void_p(pm),
+                 T * T, float("-inf"), c_void_p(py2))
+    bd2, pd2, _ = dev.put(np.full(n, -3.0), dt, offset=offset)
+    dev.lib.call("ginn_hip_scaled_masked_softmax_bwd", dev.ctx, dt, T, T * batch, c_void_p(pg), c_void_p(py2), scale,
+                 c_void_p(pm), T * T, c_void_p(pd2))
+    dev.sync()
+    get = lambda b: dev.get(b, (n,), offset=offset)
+    np.testing.assert_array_equal(get(bx2), get(bx1))
+    np.testing.assert_array_equal(get(by2), get(by1))
+    d1, d2 = get(bd1), get(bd2)
+    if dt == capi.F16:
+        # A few results per million may differ in the last bit: where a product is converted to half, the
+        # compiler emits one instruction that rounds once (v_fma_mixlo_f16) in one kernel and a multiplication
+        # in fp32 followed by a conversion, which round twice, in the other.
+        differ = d1 != d2
+        assert differ.mean() <= 2e-5
+        ulp = np.spacing(np.maximum(np.abs(d1[differ]), np.abs(d2[differ])).astype(np.float16)).astype(np.float32)
+        assert np.all(np.abs(d1[differ] - d2[differ]) <= ulp)
+    else:
+        np.testing.assert_array_equal(d2, d1)
+    # and against numpy: softmax over the rows of every column of the scaled, masked scores
+    from gpu_util import TOL
+    xs = np.where(np.tile(mask, (1, batch)) != 0, x.astype(np.float64) * scale, -np.inf)
+    e = np.exp(xs - xs.max(axis=0, keepdims=True))
+    want_y = e / e.sum(axis=0, keepdims=True)
+    got_y = get(by2).reshape(x.shape, order="F")
+    assert rel_fro(got_y, want_y) <= TOL[dt]
+    g = dy.astype(np.float64)
+    want_d = scale * np.where(np.tile(mask, (1, batch)) != 0, want_y * (g - (want_y * g).sum(axis=0, keepdims=True)), 0)
+    assert rel_fro(get(bd2).reshape(x.shape, order="F"), want_d) <= TOL[dt] * 2
+
+
+def test_scaled_masked_softmax_arguments(dev):
+    t = dev.torch
+    buf = t.zeros(256, device="cuda")
+    p, q = c_void_p(buf.data_ptr()), c_void_p(buf.data_ptr() + 512)
+    bad = [
+        ("ginn_hip_scaled_masked_softmax_fwd", (dev.ctx, capi.F32, 8, 8, p, 1.0, q, 48, 0.0, q)),   # 48 does not divide 64
+        ("ginn_hip_scaled_masked_softmax_fwd", (dev.ctx, capi.F32, 8, 8, p, 1.0, q, 64, 0.0, p)),   # y is x
+        ("ginn_hip_scaled_masked_softmax_fwd", (dev.ctx, capi.F32, 8, 8, None, 1.0, q, 64, 0.0, q)),
+        ("ginn_hip_scaled_masked_softmax_fwd", (dev.ctx, capi.F32, -8, 8, p, 1.0, q, 64, 0.0, q)),
+        ("ginn_hip_scaled_masked_softmax_bwd", (dev.ctx, capi.F32, 8, 8, p, q, 1.0, q, 0, q)),      # empty mask
+        ("ginn_hip_scaled_masked_softmax_bwd", (dev.ctx, capi.F32, 8, 8, p, q, 1.0, q, 64, p)),     # dx is dy
+        ("ginn_hip_scaled_masked_softmax_bwd", (dev.ctx, 9, 8, 8, p, q, 1.0, q, 64, c_void_p(buf.data_ptr() + 768))),
+    ]
+    for name, args in bad:
+        with pytest.raises(capi.GinnHipError):
+            dev.lib.call(name, *args)
+    dev.lib.call("ginn_hip_scaled_masked_softmax_fwd", dev.ctx, capi.F32, 0, 8, None, 1.0, None, 1, 0.0, None)
+    dev.lib.call("ginn_hip_scaled_masked_softmax_bwd", dev.ctx, capi.F32, 8, 0, None, None, 1.0, None, 1, None)
+
+
+# ---------------------------------------------------------------------------
 # GPT decoder layer through the host layer
 # ---------------------------------------------------------------------------
 
