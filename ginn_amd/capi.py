@@ -92,6 +92,9 @@ PROTOTYPES = {
     "ginn_hip_scaled_masked_softmax_bwd": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_float,
                                                    c_void_p, c_size_t, c_void_p]),
     "ginn_hip_upper_tri": (c_int, [c_void_p, c_int, c_int, c_void_p]),
+    "ginn_hip_defer_folds": (c_int, [c_void_p, c_int]),
+    "ginn_hip_flush_folds": (c_int, [c_void_p]),
+    "ginn_hip_pending_folds": (c_int, [c_void_p, POINTER(c_int)]),
     "ginn_hip_layernorm_bwd_assign": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ginn_hip_elementwise": (c_int, [c_void_p, c_int, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p, c_int]),
     "ginn_hip_fill_uniform": (c_int, [c_void_p, c_int, c_size_t, c_ulonglong, c_float, c_float, c_void_p]),

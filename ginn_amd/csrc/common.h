@@ -64,6 +64,22 @@ struct ginn_hip_pool {
   bool enabled = true;
 };
 
+// Second halves of row reductions that a caller has asked to postpone
+// (ginn_hip_defer_folds): each job folds `chunks` fp32 partial rows into up to
+// two destinations; ginn_hip_flush_folds runs all of them in one launch.
+struct ginn_hip_fold_job {
+  int dtype, rows, chunks, accumulate;
+  const float* part_a;
+  const float* part_b;
+  void* dst_a;
+  void* dst_b;
+};
+struct ginn_hip_fold_queue {
+  std::vector<ginn_hip_fold_job> jobs;
+  char* arena = nullptr;  // partial sums of the queued jobs
+  size_t arena_bytes = 0, used = 0;
+};
+
 struct ginn_hip_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
@@ -80,6 +96,7 @@ struct ginn_hip_ctx {
   hipEvent_t events[64] = {};
   int num_cus = 256;
   ginn_hip_pool pool;
+  ginn_hip_fold_queue folds;  // guarded by `mutex`
 };
 
 // A recorded sequence of launches on a context's stream.

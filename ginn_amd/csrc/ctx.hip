@@ -182,6 +182,7 @@ int ginn_hip_ctx_destroy(ginn_hip_ctx* ctx) {
   if (ctx->staging_event) (void)hipEventDestroy(ctx->staging_event);
   if (ctx->host_staging) (void)hipHostFree(ctx->host_staging);
   if (ctx->workspace) (void)hipFree(ctx->workspace);
+  if (ctx->folds.arena) (void)hipFree(ctx->folds.arena);
   pool_release_cached(ctx->pool);
   if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
@@ -202,6 +203,7 @@ int ginn_hip_ctx_stream(const ginn_hip_ctx* ctx, void** stream) {
 
 int ginn_hip_sync(ginn_hip_ctx* ctx) {
   GH_CHECK_ARG(ctx, "ginn_hip_sync: ctx is NULL");
+  if (int rc = ginn_hip_flush_folds(ctx)) return rc;  // postponed folds belong to what the caller waits for
   GH_HIP(hipStreamSynchronize(ctx->stream));
   return kOk;
 }

@@ -390,18 +390,16 @@ int ginn_hip_affine_bwd_pre(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
   const bool vec = vec8_ok({bias_src, Y, pre, dpre}, {static_cast<size_t>(m)});
   const rowred::Plan plan = rowred::plan(m, n, ctx->num_cus, ctx->workspace_bytes, 1, vec ? 8 : 1);
   GH_CHECK_ARG(plan.chunks >= 1, "ginn_hip_affine_bwd_pre: workspace too small for m=%d", m);
-  float* partial = dbias ? static_cast<float*>(ctx->workspace) : nullptr;
+  rowred::Partials room{nullptr, false};
+  if (dbias) room = rowred::take_partials(ctx, static_cast<size_t>(plan.chunks) * m * sizeof(float));
+  float* partial = room.base;
   const dim3 grid(plan.row_blocks, plan.chunks);
   GH_DISPATCH_DTYPE_V(dtype, vec, (affine_bwd_pre_kernel<T, V><<<grid, rowred::kBlock, 0, ctx->stream>>>(
       bias_act, m, n, plan.cols_per_chunk, static_cast<const T::storage*>(bias_src),
       static_cast<const T::storage*>(Y), static_cast<const T::storage*>(pre),
       static_cast<T::storage*>(dpre), partial)));
   GH_HIP(hipGetLastError());
-  if (dbias) {
-    GH_DISPATCH_DTYPE(dtype, (rowred::fold_rows_kernel<T><<<plan.fold_blocks, rowred::kFoldBlock, 0, ctx->stream>>>(
-        m, plan.chunks, partial, nullptr, static_cast<T::storage*>(dbias), nullptr, 1)));
-    GH_HIP(hipGetLastError());
-  }
+  if (dbias) return rowred::finish(ctx, {dtype, m, plan.chunks, 1, partial, nullptr, dbias, nullptr}, room.deferred);
   return kOk;
 }
 

@@ -415,15 +415,13 @@ int ginn_hip_row_sum(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols
   const bool vec = vec8_ok({x}, {static_cast<size_t>(rows)});
   const rowred::Plan plan = rowred::plan(rows, cols, ctx->num_cus, ctx->workspace_bytes, 1, vec ? 8 : 1);
   GH_CHECK_ARG(plan.chunks >= 1, "ginn_hip_row_sum: workspace too small for %d rows", rows);
-  float* partial = static_cast<float*>(ctx->workspace);
+  const rowred::Partials room = rowred::take_partials(ctx, static_cast<size_t>(plan.chunks) * rows * sizeof(float));
+  float* partial = room.base;
   GH_DISPATCH_DTYPE_V(dtype, vec, (row_sum_partial_kernel<T, V><<<dim3(plan.row_blocks, plan.chunks), rowred::kBlock,
                                                                 0, ctx->stream>>>(
       rows, cols, plan.cols_per_chunk, static_cast<const T::storage*>(x), partial)));
   GH_HIP(hipGetLastError());
-  GH_DISPATCH_DTYPE(dtype, (rowred::fold_rows_kernel<T><<<plan.fold_blocks, rowred::kFoldBlock, 0, ctx->stream>>>(
-      rows, plan.chunks, partial, nullptr, static_cast<T::storage*>(dst), nullptr, accumulate)));
-  GH_HIP(hipGetLastError());
-  return kOk;
+  return rowred::finish(ctx, {dtype, rows, plan.chunks, accumulate, partial, nullptr, dst, nullptr}, room.deferred);
 }
 
 int ginn_hip_sum_all(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n, const void* x, float scale, void* dst) {

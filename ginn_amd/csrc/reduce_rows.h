@@ -87,13 +87,12 @@ __device__ __forceinline__ void combine_v(float (&v)[V], float* red) {
 constexpr int kFoldBlock = 1024;
 constexpr int kFoldSlices = kFoldBlock / kRowsPerBlock;
 template <typename T>
-__global__ __launch_bounds__(kFoldBlock) void fold_rows_kernel(int rows, int chunks, const float* __restrict__ part_a,
-                                                               const float* __restrict__ part_b,
-                                                               typename T::storage* dst_a, typename T::storage* dst_b,
-                                                               int accumulate) {
-  __shared__ float red[2][kFoldSlices][kRowsPerBlock];
+__device__ __forceinline__ void fold_rows_block(int block, int rows, int chunks, const float* __restrict__ part_a,
+                                                const float* __restrict__ part_b, typename T::storage* dst_a,
+                                                typename T::storage* dst_b, int accumulate,
+                                                float (*red)[kFoldSlices][kRowsPerBlock]) {
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-  const int r = blockIdx.x * kRowsPerBlock + tx;
+  const int r = block * kRowsPerBlock + tx;
   float sa = 0.f, sb = 0.f;
   if (r < rows) {
 #pragma unroll 4
@@ -116,6 +115,33 @@ __global__ __launch_bounds__(kFoldBlock) void fold_rows_kernel(int rows, int chu
     if (dst_b) dst_b[r] = from_float<T>((accumulate ? to_float<T>(dst_b[r]) : 0.f) + sb);
   }
 }
+
+template <typename T>
+__global__ __launch_bounds__(kFoldBlock) void fold_rows_kernel(int rows, int chunks, const float* __restrict__ part_a,
+                                                               const float* __restrict__ part_b,
+                                                               typename T::storage* dst_a, typename T::storage* dst_b,
+                                                               int accumulate) {
+  __shared__ float red[2][kFoldSlices][kRowsPerBlock];
+  fold_rows_block<T>(blockIdx.x, rows, chunks, part_a, part_b, dst_a, dst_b, accumulate, red);
+}
+
+// ---- who folds, and when ----------------------------------------------------
+// A row-reduction entry point asks for room for its partial sums and hands the
+// fold over:
+//   Partials p = take_partials(ctx, bytes);      (ctx->mutex held)
+//   ... launch the kernel that writes p.base ...
+//   finish(ctx, job, p.deferred);
+// Normally the room is the context's workspace and finish() launches
+// fold_rows_kernel.  While the calling thread has asked for it
+// (ginn_hip_defer_folds) the partial sums go to an area of their own, the job
+// is queued, and flush_folds() folds everything queued in one launch.
+struct Partials {
+  float* base;
+  bool deferred;
+};
+Partials take_partials(ginn_hip_ctx* ctx, size_t bytes);
+int finish(ginn_hip_ctx* ctx, const ginn_hip_fold_job& job, bool deferred);
+int flush_folds(ginn_hip_ctx* ctx);  // ctx->mutex held
 
 }  // namespace rowred
 }  // namespace ginn_hip

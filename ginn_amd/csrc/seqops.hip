@@ -478,18 +478,15 @@ int ginn_hip_cwise_prod_add_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int row
   const bool vec = vec8_ok({dy, a, b, da}, {static_cast<size_t>(rows)});
   const rowred::Plan plan = rowred::plan(rows, cols, ctx->num_cus, ctx->workspace_bytes, 2, vec ? 8 : 1);
   GH_CHECK_ARG(plan.chunks >= 1, "ginn_hip_cwise_prod_add_bwd: workspace too small for %d rows", rows);
-  float* part_b = static_cast<float*>(ctx->workspace);
+  const rowred::Partials room = rowred::take_partials(ctx, 2 * static_cast<size_t>(plan.chunks) * rows * sizeof(float));
+  float* part_b = room.base;
   float* part_c = part_b + static_cast<size_t>(plan.chunks) * rows;
   GH_DISPATCH_DTYPE_V(dtype, vec, (cwise_prod_add_bwd_bcast_kernel<T, V><<<dim3(plan.row_blocks, plan.chunks),
                                                                            rowred::kBlock, 0, ctx->stream>>>(
       rows, cols, plan.cols_per_chunk, static_cast<const T::storage*>(dy), static_cast<const T::storage*>(a),
       static_cast<const T::storage*>(b), multiplier_bias, static_cast<T::storage*>(da), part_b, part_c)));
   GH_HIP(hipGetLastError());
-  if (db || dc) {
-    GH_DISPATCH_DTYPE(dtype, (rowred::fold_rows_kernel<T><<<plan.fold_blocks, rowred::kFoldBlock, 0, ctx->stream>>>(
-        rows, plan.chunks, part_b, part_c, static_cast<T::storage*>(db), static_cast<T::storage*>(dc), 1)));
-    GH_HIP(hipGetLastError());
-  }
+  if (db || dc) return rowred::finish(ctx, {dtype, rows, plan.chunks, 1, part_b, part_c, db, dc}, room.deferred);
   return kOk;
 }
 

@@ -760,6 +760,7 @@ class LevelExecutor {
   // level; reset_grad() must have run (ginn/node.h:237-254).
   LevelExecutor& backward(double loss_coeff = 1) {
     seed_sink(loss_coeff);
+    internal::FoldWindow folds;  // row sums into leaf gradients are folded once, at the end
     if (frozen_) {
       if (fused_ready_) {
         run_fused(kBackward);
@@ -770,6 +771,7 @@ class LevelExecutor {
         }
       }
       for (BaseNode* n : lazy_direct_) n->clear_lazy_zero();  // all taken already, unless a node returned early
+      folds.close();
       return *this;
     }
     cursor_ = 0;
@@ -796,6 +798,7 @@ class LevelExecutor {
       }
       flush(kBackward, step);
     }
+    folds.close();
     std::sort(taken_by_plans_.begin(), taken_by_plans_.end());
     lazy_direct_.clear();
     for (BaseNode* n : lazy_)

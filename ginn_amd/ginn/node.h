@@ -10,6 +10,7 @@
 #include <memory>
 #include <string>
 #include <type_traits>
+#include <algorithm>
 #include <atomic>
 #include <cstdint>
 #include <utility>
@@ -307,6 +308,65 @@ inline std::atomic<size_t>& lazy_grad_settles() {
   static std::atomic<size_t> n{0};
   return n;
 }
+// Open while Graph::backward() / LevelExecutor::backward() runs on this thread.
+// A row sum into the gradient of a leaf node (a bias, a LayerNorm scale) is two
+// launches, partial sums and their fold; nothing reads such a gradient before
+// the pass ends, so while a window is open the nodes postpone those folds
+// (ginn_hip_defer_folds) and the pass runs them all as one launch at its end.
+class FoldWindow {
+  static int& depth() {
+    thread_local int d = 0;
+    return d;
+  }
+  static std::vector<ginn_hip_ctx*>& touched() {
+    thread_local std::vector<ginn_hip_ctx*> v;
+    return v;
+  }
+
+ public:
+  FoldWindow() { ++depth(); }
+  FoldWindow(const FoldWindow&) = delete;
+  FoldWindow& operator=(const FoldWindow&) = delete;
+  ~FoldWindow() {
+    if (--depth() == 0 && !touched().empty()) {  // left by an exception: nothing stays queued
+      for (ginn_hip_ctx* c : touched()) (void)ginn_hip_flush_folds(c);
+      touched().clear();
+    }
+  }
+  static bool open() { return depth() > 0; }
+  static void note(ginn_hip_ctx* ctx) {
+    auto& v = touched();
+    if (std::find(v.begin(), v.end(), ctx) == v.end()) v.push_back(ctx);
+  }
+  // The end of the pass: the outermost window folds what was postponed.
+  void close() {
+    if (depth() != 1) return;
+    std::vector<ginn_hip_ctx*> v;
+    v.swap(touched());
+    for (ginn_hip_ctx* c : v) GINN_HIP_CALL(ginn_hip_flush_folds(c));
+  }
+};
+
+// Around one library call whose row sums go into the gradient of `target`.
+class PostponeFolds {
+  ginn_hip_ctx* ctx_ = nullptr;
+
+ public:
+  template <typename... Targets>
+  PostponeFolds(ginn_hip_ctx* ctx, const Targets&... targets) {
+    const bool leaves = (... && targets.inputs().empty());
+    if (FoldWindow::open() && leaves && ginn_hip_defer_folds(ctx, 1) == 0) {
+      ctx_ = ctx;
+      FoldWindow::note(ctx);
+    }
+  }
+  PostponeFolds(const PostponeFolds&) = delete;
+  PostponeFolds& operator=(const PostponeFolds&) = delete;
+  ~PostponeFolds() {
+    if (ctx_) (void)ginn_hip_defer_folds(ctx_, 0);
+  }
+};
+
 // While set, every gradient whose flag is taken is noted here (the level
 // executor tells apart the flags that recorded launches consume).
 inline std::vector<BaseNode*>*& lazy_take_log() {
@@ -409,8 +469,10 @@ class Graph {
     } else {
       GINN_THROW("Unexpected scalar type in sink node!");
     }
+    internal::FoldWindow folds;
     for (auto it = list_.rbegin(); it != list_.rend(); ++it)
       if ((*it)->has_grad()) (*it)->backward();
+    folds.close();
     return *this;
   }
 

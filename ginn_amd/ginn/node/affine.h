@@ -66,6 +66,7 @@ class AffineNode : public BaseDataNode<Scalar> {
     if (!identity) dpreactiv_.resize(grad().shape());
     auto& bias = ins_.back();
     const Size m = grad().rows(), n = grad().cols();
+    PostponeFolds later(ctx_of(grad()), *bias);  // the bias gradient is complete when the pass ends
     GINN_HIP_CALL(ginn_hip_affine_bwd_pre(ctx_of(grad()), dtype_of<Scalar>(), nonlin_->code(),
                                           static_cast<int>(m), static_cast<int>(n), grad().data(),
                                           value().data(), preactiv_.size() > 0 ? preactiv_.data() : nullptr,

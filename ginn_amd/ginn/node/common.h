@@ -236,6 +236,7 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
   }
   void backward_() override {
     auto& a = a_->value();
+    internal::PostponeFolds later(internal::ctx_of(a), *b_, *c_);  // scale / shift gradients: complete at the pass's end
     GINN_HIP_CALL(ginn_hip_cwise_prod_add_bwd(
         internal::ctx_of(a), dtype_of<Scalar>(), static_cast<int>(a.rows()), static_cast<int>(a.cols()),
         grad().data(), a.data(), b_->value().data(), multiplier_bias_, broadcast_ ? 1 : 0,

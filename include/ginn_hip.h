@@ -344,6 +344,27 @@ int ginn_hip_col_broadcast(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows,
 int ginn_hip_row_sum(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols,
                      const void* x, void* dst, int accumulate);
 
+/* Row sums are two launches: partial sums per chunk of columns, then a fold of
+ * the chunks.  A backward pass makes one such pair per bias gradient
+ * (AffineNode::backward_, ginn/node/affine.h:117-122) and per scale / shift
+ * gradient of CwiseProdAdd (ginn/node/common.h:296-316); the reference does
+ * each as one Eigen reduction.  A caller that does not read those sums before
+ * the end of the pass may postpone the folds and run them as one launch:
+ *   ginn_hip_defer_folds(ctx, 1);   folds of row reductions that THIS host
+ *                                   thread starts from now on are queued
+ *                                   (ginn_hip_affine_bwd_pre's dbias,
+ *                                   ginn_hip_cwise_prod_add_bwd's db / dc,
+ *                                   ginn_hip_row_sum); calls nest
+ *   ginn_hip_defer_folds(ctx, 0);   back to folding at once (queued folds stay queued)
+ *   ginn_hip_flush_folds(ctx);      one launch for everything queued on ctx
+ * Until the flush the destinations hold their old values.  The queue also
+ * empties by itself when its 8 MiB of partial sums are full, when two queued
+ * folds would add into one destination, and in ginn_hip_sync.  The sums are
+ * the same bits as without postponing. */
+int ginn_hip_defer_folds(ginn_hip_ctx* ctx, int on);
+int ginn_hip_flush_folds(ginn_hip_ctx* ctx);
+int ginn_hip_pending_folds(ginn_hip_ctx* ctx, int* count);
+
 /* dst[0] = scale * sum_i x[i]; SumNode / MeanNode forward
  * (ginn/node/reduce.h:30-75,138-159). */
 int ginn_hip_sum_all(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,

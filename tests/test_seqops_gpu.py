@@ -269,6 +269,68 @@ def test_scaled_masked_softmax_arguments(dev):
 
 
 # ---------------------------------------------------------------------------
+# postponed folds of row sums
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_postponed_folds_give_the_same_sums(dev, dt):
+    """ginn_hip_defer_folds / ginn_hip_flush_folds: the second launch of every row
+    reduction started meanwhile waits, the destinations keep their old values,
+    one launch then folds all of them to the bits of the unpostponed calls; two
+    folds into one destination are not put into one launch."""
+    from gpu_util import round_to
+    rng = np.random.default_rng(11)
+    shapes = [(768, 520), (40, 33), (1024, 64)]
+    xs = [round_to(rng.standard_normal(s), dt) for s in shapes]
+    old = [round_to(rng.standard_normal(s[0]), dt) for s in shapes]
+
+    def row_sums(postpone):
+        outs = []
+        for x, o in zip(xs, old):
+            bx, px, _ = dev.put(x, dt)
+            bo, po, _ = dev.put(o, dt)
+            outs.append((bx, bo, px, po, x.shape))
+        if postpone:
+            dev.lib.call("ginn_hip_defer_folds", dev.ctx, 1)
+        for bx, bo, px, po, (r, c) in outs:
+            dev.lib.call("ginn_hip_row_sum", dev.ctx, dt, r, c, c_void_p(px), c_void_p(po), 1)
+        if postpone:
+            dev.lib.call("ginn_hip_defer_folds", dev.ctx, 0)
+            n = ctypes.c_int(-1)
+            dev.lib.call("ginn_hip_pending_folds", dev.ctx, ctypes.byref(n))
+            assert n.value == len(shapes)
+            for (bx, bo, px, po, (r, c)), o in zip(outs, old):   # nothing folded yet
+                np.testing.assert_array_equal(dev.get(bo, (r,)), o)
+            dev.lib.call("ginn_hip_flush_folds", dev.ctx)
+            dev.lib.call("ginn_hip_pending_folds", dev.ctx, ctypes.byref(n))
+            assert n.value == 0
+        dev.sync()
+        return [dev.get(bo, (r,)) for bx, bo, px, po, (r, c) in outs]
+
+    plain, later = row_sums(False), row_sums(True)
+    for a, b, x, o in zip(plain, later, xs, old):
+        np.testing.assert_array_equal(b, a)
+        from gpu_util import TOL
+        assert rel_fro(a, x.astype(np.float64).sum(axis=1) + o) <= TOL[dt]
+
+    # two sums into one destination: the second one folds the first before it queues itself
+    bx, px, _ = dev.put(xs[0], dt)
+    bo, po, _ = dev.put(np.zeros(shapes[0][0]), dt)
+    dev.lib.call("ginn_hip_defer_folds", dev.ctx, 1)
+    for _ in range(2):
+        dev.lib.call("ginn_hip_row_sum", dev.ctx, dt, shapes[0][0], shapes[0][1], c_void_p(px), c_void_p(po), 1)
+    n = ctypes.c_int(-1)
+    dev.lib.call("ginn_hip_pending_folds", dev.ctx, ctypes.byref(n))
+    assert n.value == 1
+    dev.lib.call("ginn_hip_defer_folds", dev.ctx, 0)
+    dev.sync()  # waits for the postponed fold as well
+    once = round_to(xs[0].astype(np.float64).sum(axis=1), dt)
+    assert rel_fro(dev.get(bo, (shapes[0][0],)), 2.0 * once) <= TOL[dt]
+    with pytest.raises(capi.GinnHipError):
+        dev.lib.call("ginn_hip_defer_folds", dev.ctx, 0)   # switched off more often than on
+
+
+# ---------------------------------------------------------------------------
 # GPT decoder layer through the host layer
 # ---------------------------------------------------------------------------
 
