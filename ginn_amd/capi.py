@@ -77,6 +77,9 @@ PROTOTYPES = {
     "ginn_hip_add_scalar_bcast": (c_int, [c_void_p, c_int, c_size_t, c_void_p, c_float, c_void_p]),
     "ginn_hip_pick_nls_fwd": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ginn_hip_pick_nls_bwd": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_pick_nls_fwd_stats": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_pick_nls_bwd_stats": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_int]),
     "ginn_hip_pick_nls_bwd_assign": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ginn_hip_layernorm_fwd": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p]),
     "ginn_hip_layernorm_bwd": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),

@@ -214,6 +214,7 @@ __global__ __launch_bounds__(kBlock) void pick_nls_fwd_kernel(int rows, int cols
                                                               const typename T::storage* __restrict__ x,
                                                               const int* __restrict__ idx,
                                                               typename T::storage* __restrict__ smax,
+                                                              float* __restrict__ stats,
                                                               typename T::storage* __restrict__ out) {
   const int lane = threadIdx.x & 63;
   const int wave = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
@@ -237,12 +238,16 @@ __global__ __launch_bounds__(kBlock) void pick_nls_fwd_kernel(int rows, int cols
     }
     sum = wave_sum(sum);
     const float inv = 1.f / sum;
-    for (int r = lane * V; r < rows; r += 64 * V) {
+    for (int r = lane * V; smax && r < rows; r += 64 * V) {
       float v[V];
       ld<T, V>(x + base + r, v);
 #pragma unroll
       for (int e = 0; e < V; ++e) v[e] = softmax_exp<T>(v[e] - mx) * inv;
       st<T, V>(smax + base + r, v);
+    }
+    if (stats && lane == 0) {
+      stats[2 * c] = mx;
+      stats[2 * c + 1] = inv;
     }
     if (lane == 0) {
       // -log of the value as stored, as the reference picks from the stored
@@ -259,6 +264,7 @@ __global__ __launch_bounds__(kBlock) void pick_nls_fwd_regs_kernel(int rows, int
                                                                    const typename T::storage* __restrict__ x,
                                                                    const int* __restrict__ idx,
                                                                    typename T::storage* __restrict__ smax,
+                                                                   float* __restrict__ stats,
                                                                    typename T::storage* __restrict__ out) {
   const int lane = threadIdx.x & 63;
   const int wave = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
@@ -271,7 +277,11 @@ __global__ __launch_bounds__(kBlock) void pick_nls_fwd_regs_kernel(int rows, int
     if (lane == 0) picked_x = to_float<T>(x[base + idx[c]]);
     float mx, inv;
     col.softmax(mx, inv);
-    col.store(smax + base, rows, lane);
+    if (smax) col.store(smax + base, rows, lane);
+    if (stats && lane == 0) {
+      stats[2 * c] = mx;
+      stats[2 * c + 1] = inv;
+    }
     if (lane == 0) {
       const float picked = to_float<T>(from_float<T>(softmax_exp<T>(picked_x - mx) * inv));
       out[c] = from_float<T>(-logf(picked));
@@ -302,6 +312,41 @@ __global__ __launch_bounds__(kBlock) void pick_nls_bwd_kernel(int rows, int cols
 #pragma unroll
     for (int e = 0; e < V; ++e) v[e] += sm[e] * g - (e == hot ? g : 0.f);
     st<T, V>(dx + i, v);
+  }
+}
+
+// The same from the logits and the column statistics the forward kernel left
+// (maximum, 1 / sum of exponentials) instead of the stored softmax: the softmax
+// is rebuilt, rounded to the storage type as the stored one was.  One wave per column.
+template <typename T, int V>
+__global__ __launch_bounds__(kBlock) void pick_nls_bwd_stats_kernel(int rows, int cols,
+                                                                    const typename T::storage* __restrict__ x,
+                                                                    const float* __restrict__ stats,
+                                                                    const int* __restrict__ idx,
+                                                                    const typename T::storage* __restrict__ dout,
+                                                                    typename T::storage* dx, int accumulate) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * (kBlock / 64);
+  for (int c = wave; c < cols; c += nwaves) {
+    const size_t base = static_cast<size_t>(c) * rows;
+    const float mx = stats[2 * c], inv = stats[2 * c + 1];
+    const float g = to_float<T>(dout[c]);
+    const int picked = idx[c];
+    for (int r = lane * V; r < rows; r += 64 * V) {
+      float v[V], old[V];
+      ld<T, V>(x + base + r, v);
+#pragma unroll
+      for (int e = 0; e < V; ++e) old[e] = 0.f;
+      if (accumulate) ld<T, V>(dx + base + r, old);
+      const int hot = picked - r;
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float sm = to_float<T>(from_float<T>(softmax_exp<T>(v[e] - mx) * inv));
+        v[e] = old[e] + (sm * g - (e == hot ? g : 0.f));
+      }
+      st<T, V>(dx + base + r, v);
+    }
   }
 }
 
@@ -459,12 +504,12 @@ int ginn_hip_add_scalar_bcast(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
   return kOk;
 }
 
-int ginn_hip_pick_nls_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* x, const int* idx,
-                          void* smax, void* out) {
-  GH_CHECK_ARG(ctx, "ginn_hip_pick_nls_fwd: ctx is NULL");
-  GH_CHECK_ARG(rows >= 1 && cols >= 0, "ginn_hip_pick_nls_fwd: bad dimension");
+static int pick_nls_fwd(const char* who, ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* x,
+                        const int* idx, void* smax, float* stats, void* out) {
+  GH_CHECK_ARG(ctx, "%s: ctx is NULL", who);
+  GH_CHECK_ARG(rows >= 1 && cols >= 0, "%s: bad dimension", who);
   if (cols == 0) return kOk;
-  GH_CHECK_ARG(x && idx && smax && out, "ginn_hip_pick_nls_fwd: NULL pointer");
+  GH_CHECK_ARG(x && idx && (smax || stats) && out, "%s: NULL pointer", who);
   GH_HIP(hipSetDevice(ctx->device));
   const unsigned grid = grid_for(cols, kBlock / 64, ctx->num_cus);
   const bool vec = vec8_ok({x, smax}, {static_cast<size_t>(rows)});
@@ -472,14 +517,44 @@ int ginn_hip_pick_nls_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int
   if (vec && vectors) {
     GH_DISPATCH_COLUMN_VECTORS(vectors, {
       GH_DISPATCH_DTYPE(dtype, (pick_nls_fwd_regs_kernel<T, I><<<grid, kBlock, 0, ctx->stream>>>(
-          rows, cols, static_cast<const T::storage*>(x), idx, static_cast<T::storage*>(smax),
+          rows, cols, static_cast<const T::storage*>(x), idx, static_cast<T::storage*>(smax), stats,
           static_cast<T::storage*>(out))));
     });
     GH_HIP(hipGetLastError());
     return kOk;
   }
   GH_DISPATCH_DTYPE_V(dtype, vec, (pick_nls_fwd_kernel<T, V><<<grid, kBlock, 0, ctx->stream>>>(
-      rows, cols, static_cast<const T::storage*>(x), idx, static_cast<T::storage*>(smax), static_cast<T::storage*>(out))));
+      rows, cols, static_cast<const T::storage*>(x), idx, static_cast<T::storage*>(smax), stats,
+      static_cast<T::storage*>(out))));
+  GH_HIP(hipGetLastError());
+  return kOk;
+}
+
+int ginn_hip_pick_nls_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* x, const int* idx,
+                          void* smax, void* out) {
+  GH_CHECK_ARG(smax || cols == 0, "ginn_hip_pick_nls_fwd: NULL pointer");
+  return pick_nls_fwd("ginn_hip_pick_nls_fwd", ctx, dtype, rows, cols, x, idx, smax, nullptr, out);
+}
+
+int ginn_hip_pick_nls_fwd_stats(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* x,
+                                const int* idx, float* stats, void* out) {
+  GH_CHECK_ARG(stats || cols == 0, "ginn_hip_pick_nls_fwd_stats: NULL pointer");
+  return pick_nls_fwd("ginn_hip_pick_nls_fwd_stats", ctx, dtype, rows, cols, x, idx, nullptr, stats, out);
+}
+
+int ginn_hip_pick_nls_bwd_stats(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* x,
+                                const float* stats, const int* idx, const void* dout, void* dx, int accumulate) {
+  GH_CHECK_ARG(ctx, "ginn_hip_pick_nls_bwd_stats: ctx is NULL");
+  GH_CHECK_ARG(rows >= 1 && cols >= 0, "ginn_hip_pick_nls_bwd_stats: bad dimension");
+  if (cols == 0) return kOk;
+  GH_CHECK_ARG(x && stats && idx && dout && dx, "ginn_hip_pick_nls_bwd_stats: NULL pointer");
+  GH_CHECK_ARG(x != dx, "ginn_hip_pick_nls_bwd_stats: dx must not be x");
+  GH_HIP(hipSetDevice(ctx->device));
+  const bool vec = vec8_ok({x, dx}, {static_cast<size_t>(rows)});
+  const unsigned grid = grid_for(cols, kBlock / 64, ctx->num_cus);
+  GH_DISPATCH_DTYPE_V(dtype, vec, (pick_nls_bwd_stats_kernel<T, V><<<grid, kBlock, 0, ctx->stream>>>(
+      rows, cols, static_cast<const T::storage*>(x), stats, idx, static_cast<const T::storage*>(dout),
+      static_cast<T::storage*>(dx), accumulate)));
   GH_HIP(hipGetLastError());
   return kOk;
 }

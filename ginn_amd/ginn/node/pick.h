@@ -92,31 +92,36 @@ GINN_MAKE_SCALAR_FORWARDING_FACTORY(PickSoftmax);
 
 // value[0, c] = -log softmax(x)[index[c], c]; backward dx += softmax * dy
 // (broadcast down the column), dx[index[c], c] -= dy[c]
-// (ginn/node/pick.h:203-248).  Forward and backward are one kernel each.
+// (ginn/node/pick.h:203-248).  Forward and backward are one kernel each.  The
+// reference keeps the softmax matrix for backward; here forward keeps the
+// maximum and the sum of exponentials of every column (two floats) and backward
+// rebuilds the softmax from the input, rounded as it would have been stored:
+// the same gradient, and forward writes [1 x cols] instead of [rows x cols].
 template <typename Scalar>
 class PickNegLogSoftmaxNode : public PickSoftmaxNode<Scalar> {
   using PickSoftmaxNode<Scalar>::in_;
-  using PickSoftmaxNode<Scalar>::smax_;
   using PickNode<Scalar>::index_;
+  Tensor<float> stats_;  // per column: maximum, 1 / sum of exp(x - maximum)
 
   void forward_() override {
     internal::require_gpu(this->dev(), "PickNegLogSoftmax");
     auto& x = in_->value();
     this->check_index(x);
-    smax_.move_to(this->dev());
-    smax_.resize(x.shape2());
+    stats_.move_to(this->dev());
+    stats_.resize(2, x.cols());
     value().resize(1, x.cols());
-    GINN_HIP_CALL(ginn_hip_pick_nls_fwd(internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()),
-                                        static_cast<int>(x.cols()), x.data(), index_->value().data(),
-                                        smax_.data(), value().data()));
+    GINN_HIP_CALL(ginn_hip_pick_nls_fwd_stats(internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()),
+                                              static_cast<int>(x.cols()), x.data(), index_->value().data(),
+                                              stats_.data(), value().data()));
   }
   void backward_() override {
     if (!in_->has_grad()) return;
     auto& x = in_->value();
     const bool fresh = in_->take_lazy_zero();
-    GINN_HIP_CALL((fresh ? ginn_hip_pick_nls_bwd_assign : ginn_hip_pick_nls_bwd)(
-        internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()), static_cast<int>(x.cols()),
-        smax_.data(), index_->value().data(), grad().data(), in_->grad().data()));
+    GINN_HIP_CALL(ginn_hip_pick_nls_bwd_stats(internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()),
+                                              static_cast<int>(x.cols()), x.data(), stats_.data(),
+                                              index_->value().data(), grad().data(), in_->grad().data(),
+                                              fresh ? 0 : 1));
   }
 
  public:

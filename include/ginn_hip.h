@@ -384,6 +384,18 @@ int ginn_hip_pick_nls_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows,
 int ginn_hip_pick_nls_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows,
                           int cols, const void* smax, const int* idx,
                           const void* dout, void* dx);
+/* The pair without the softmax matrix: forward leaves stats[2 c] = maximum of
+ * column c and stats[2 c + 1] = 1 / sum_r exp(x[r, c] - maximum) (fp32, DEVICE
+ * array of 2 * cols), backward rebuilds softmax(x) from them, rounded to the
+ * storage type as ginn_hip_pick_nls_fwd would have stored it, and assigns
+ * (accumulate == 0) or adds.  x must still hold the forward pass's values. */
+int ginn_hip_pick_nls_fwd_stats(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                                int rows, int cols, const void* x,
+                                const int* idx, float* stats, void* out);
+int ginn_hip_pick_nls_bwd_stats(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                                int rows, int cols, const void* x,
+                                const float* stats, const int* idx,
+                                const void* dout, void* dx, int accumulate);
 /* The same with `=` in place of `+=`: what the backward pass of
  * ginn/node/pick.h:226-236 leaves in a gradient that reset_grad() had just
  * zeroed (ginn/node.h:218-222), without reading the zeros. */

@@ -439,3 +439,37 @@ def test_pick_neg_log_softmax(dev, dt, rows, cols):
     onehot[labels, np.arange(cols)] = 1.0
     want_dx = dx0 + (sm.astype(np.float64) - onehot) * dout.astype(np.float64)
     assert rel_fro(dev.get(b_dx, (rows, cols)), want_dx) <= TOL[dt] * 2
+
+    # The pair that keeps two numbers per column instead of the softmax matrix: the same loss bits; the
+    # gradient, adding and assigning, as from the stored softmax (for half storage a few results per
+    # million may differ in the last bit: the product with 1 / sum is rounded to half by one instruction
+    # in one kernel and by two in the other).
+    b_t = torch.full((2 * cols,), float("nan"), device="cuda", dtype=torch.float32)
+    b_o2, p_o2, _ = dev.put(np.full((1, cols), np.nan, np.float32), dt)
+    dev.lib.call("ginn_hip_pick_nls_fwd_stats", dev.ctx, dt, rows, cols, ctypes.c_void_p(p_x),
+                 ctypes.c_void_p(idx.data_ptr()), ctypes.c_void_p(b_t.data_ptr()), ctypes.c_void_p(p_o2))
+    for accumulate in (1, 0):
+        b_dx2, p_dx2, _ = dev.put(dx0, dt)
+        dev.lib.call("ginn_hip_pick_nls_bwd_stats", dev.ctx, dt, rows, cols, ctypes.c_void_p(p_x),
+                     ctypes.c_void_p(b_t.data_ptr()), ctypes.c_void_p(idx.data_ptr()), ctypes.c_void_p(p_d),
+                     ctypes.c_void_p(p_dx2), accumulate)
+        b_ref, p_ref, _ = dev.put(dx0, dt)
+        dev.lib.call("ginn_hip_pick_nls_bwd" if accumulate else "ginn_hip_pick_nls_bwd_assign", dev.ctx, dt, rows,
+                     cols, ctypes.c_void_p(p_s), ctypes.c_void_p(idx.data_ptr()), ctypes.c_void_p(p_d),
+                     ctypes.c_void_p(p_ref))
+        dev.sync()
+        got, ref = dev.get(b_dx2, (rows, cols)), dev.get(b_ref, (rows, cols))
+        if dt == capi.F16:
+            differ = got != ref
+            assert differ.mean() <= 1e-4 or differ.sum() <= 1
+            ulp = np.spacing(np.maximum(np.abs(got[differ]), np.abs(ref[differ])).astype(np.float16)).astype(np.float32)
+            assert np.all(np.abs(got[differ] - ref[differ]) <= ulp)
+        else:
+            np.testing.assert_array_equal(got, ref)
+        if not accumulate:
+            assert rel_fro(got, (sm.astype(np.float64) - onehot) * dout.astype(np.float64)) <= TOL[dt] * 2
+    np.testing.assert_array_equal(dev.get(b_o2, (1, cols)).ravel(), nll)
+    stats = b_t.cpu().numpy().reshape(cols, 2)
+    np.testing.assert_allclose(stats[:, 0], x.max(axis=0), rtol=0, atol=0)
+    np.testing.assert_allclose(1.0 / stats[:, 1], np.exp(x.astype(np.float64) - x.max(axis=0)).sum(axis=0),
+                               rtol={capi.F32: 1e-5}.get(dt, 5e-3))
