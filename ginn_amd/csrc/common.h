@@ -385,6 +385,9 @@ int launch_gemm_skinny_mfma(ginn_hip_ctx* ctx, const GemmArgs& args);
 // 16-bit, 128 x 128 x 64 tiles with optional split-K: aligned shapes whose
 // 256 x 256 tiling would leave most CUs idle; kUnsupported otherwise.
 int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& args);
+// Batched 16-bit products with small, memory-bound slices (attention shapes);
+// kUnsupported for everything else (gemm_bsmall.hip).
+int launch_gemm_bsmall(ginn_hip_ctx* ctx, const GemmArgs& args);
 // Folds `splits` fp32 partial products [split][n][m] and applies the epilogue
 // of `args` (beta, bias, activation, pre-activation) into C.
 int launch_splitk_reduce(ginn_hip_ctx* ctx, const GemmArgs& args, int splits, const float* partial);

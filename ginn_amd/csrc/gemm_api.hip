@@ -54,6 +54,8 @@ int launch_gemm(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (rc != kUnsupported) return rc;
   rc = launch_gemm_fast16(ctx, a);
   if (rc != kUnsupported) return rc;
+  rc = launch_gemm_bsmall(ctx, a);
+  if (rc != kUnsupported) return rc;
   rc = launch_gemm_mid(ctx, a);
   if (rc != kUnsupported) return rc;
   return launch_gemm_generic(ctx, a);
