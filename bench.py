@@ -439,15 +439,15 @@ def other_configs(cpu):
     """The graph-level configurations of the build target, a few passes each, outside the headline's timed
     region: GPU ms per fwd+bwd pass through the frozen level executor, and the CPU oracle on one thread."""
     out = {}
-    g = bench_gpt(4, cpu, executor=6)
+    g = bench_gpt(30, cpu, executor=6)
     out["gpt_ms"], out["gpt_tflops"] = g["gpu_ms"], g["tflops"]
     if cpu:
         out["gpt_cpu_ms"] = g["cpu_ms"]
-    r = bench_mlp(20, cpu, executor=6)
+    r = bench_mlp(100, cpu, executor=6)
     out["mlp_ms"] = r["gpu_ms"]
     if cpu:
         out["mlp_cpu_ms"] = r["cpu_ms"]
-    r = bench_lstm(4, cpu, mode=23, gather=True)
+    r = bench_lstm(10, cpu, mode=23, gather=True)
     out["lstm_ms"] = r["gpu_ms"]
     if cpu:
         out["lstm_cpu_ms"] = r["cpu_ms"]

@@ -87,6 +87,12 @@ PROTOTYPES = {
                                             c_int, c_void_p]),
     "ginn_hip_cwise_prod_add_bwd": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_float,
                                             c_int, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_cwise_prod_add_bwd_assign": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_float,
+                                            c_int, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_layernorm_affine_fwd": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p,
+                                              c_float, c_void_p, c_void_p, c_void_p]),
+    "ginn_hip_layernorm_affine_bwd": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                              c_float, c_void_p, c_int, c_void_p, c_void_p]),
     "ginn_hip_permute": (c_int, [c_void_p, c_int, c_int, POINTER(c_longlong), POINTER(c_int), c_void_p, c_void_p,
                                  c_int]),
     "ginn_hip_mask_fill": (c_int, [c_void_p, c_int, c_size_t, c_size_t, c_void_p, c_float, c_void_p]),

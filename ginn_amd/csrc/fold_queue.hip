@@ -23,9 +23,9 @@ struct FoldJobs {
 };
 
 __global__ __launch_bounds__(rowred::kFoldBlock) void multi_fold_kernel(FoldJobs jobs) {
-  __shared__ float red[2][rowred::kFoldSlices][rowred::kRowsPerBlock];
+  __shared__ float red[2][rowred::kFoldSlices][rowred::kFoldRows];
   const ginn_hip_fold_job& j = jobs.job[blockIdx.y];
-  if (static_cast<int>(blockIdx.x) * rowred::kRowsPerBlock >= j.rows) return;  // whole block: no barrier is skipped
+  if (static_cast<int>(blockIdx.x) * rowred::kFoldRows >= j.rows) return;  // whole block: no barrier is skipped
   switch (j.dtype) {
     case GINN_HIP_F32:
       rowred::fold_rows_block<F32>(blockIdx.x, j.rows, j.chunks, j.part_a, j.part_b, static_cast<float*>(j.dst_a),
@@ -61,7 +61,7 @@ int flush_folds(ginn_hip_ctx* ctx) {
     int blocks = 1;
     for (size_t i = 0; i < count; ++i) {
       args.job[i] = q.jobs[first + i];
-      blocks = std::max(blocks, (args.job[i].rows + kRowsPerBlock - 1) / kRowsPerBlock);
+      blocks = std::max(blocks, (args.job[i].rows + kFoldRows - 1) / kFoldRows);
     }
     multi_fold_kernel<<<dim3(blocks, static_cast<unsigned>(count)), kFoldBlock, 0, ctx->stream>>>(args);
     GH_HIP(hipGetLastError());
@@ -114,7 +114,7 @@ int finish(ginn_hip_ctx* ctx, const ginn_hip_fold_job& job, bool deferred) {
     q.jobs.push_back(job);
     return kOk;
   }
-  const int blocks = (job.rows + kRowsPerBlock - 1) / kRowsPerBlock;
+  const int blocks = (job.rows + kFoldRows - 1) / kFoldRows;
   GH_DISPATCH_DTYPE(job.dtype, (fold_rows_kernel<T><<<blocks, kFoldBlock, 0, ctx->stream>>>(
       job.rows, job.chunks, job.part_a, job.part_b, static_cast<T::storage*>(job.dst_a),
       static_cast<T::storage*>(job.dst_b), job.accumulate)));

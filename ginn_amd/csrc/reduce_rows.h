@@ -4,7 +4,7 @@
 // a wave reads consecutive addresses either way) and a chunk of columns; its 4
 // waves take every 4th column of the chunk and combine through LDS.  Per-chunk
 // fp32 partials are folded by fold_rows_kernel, which spreads the chunks of a
-// row over 16 waves.
+// row over 64 threads.
 #ifndef GINN_HIP_REDUCE_ROWS_H
 #define GINN_HIP_REDUCE_ROWS_H
 
@@ -17,6 +17,11 @@ constexpr int kBlock = 256;
 constexpr int kRowsPerBlock = 64;
 constexpr int kSlices = kBlock / kRowsPerBlock;  // waves per block = column phases
 constexpr int kMaxChunks = 128;
+// The fold: a block of 1024 threads owns 16 rows and spreads their chunks over
+// 64 slices (the fold is pure latency: few bytes, many loads in flight).
+constexpr int kFoldBlock = 1024;
+constexpr int kFoldRows = 16;
+constexpr int kFoldSlices = kFoldBlock / kFoldRows;
 
 struct Plan {
   int row_blocks;   // grid.x of the partial kernel (64 V rows each)
@@ -30,7 +35,7 @@ inline Plan plan(int rows, int cols, int num_cus, size_t workspace_bytes, int su
   Plan p;
   const int per_block = kRowsPerBlock * rows_per_lane;
   p.row_blocks = (rows + per_block - 1) / per_block;
-  p.fold_blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+  p.fold_blocks = (rows + kFoldRows - 1) / kFoldRows;
   int chunks = (num_cus * 4 + p.row_blocks - 1) / p.row_blocks;
   if (chunks > kMaxChunks) chunks = kMaxChunks;
   if (chunks > (cols + 4 * kSlices - 1) / (4 * kSlices)) chunks = (cols + 4 * kSlices - 1) / (4 * kSlices);
@@ -81,18 +86,16 @@ __device__ __forceinline__ void combine_v(float (&v)[V], float* red) {
   __syncthreads();
 }
 
-// dst[r] (+)= sum over chunks of partial[c][r], for up to two partial arrays.
-// A block of 1024 threads owns 64 rows; its 16 waves take every 16th chunk
-// (many loads in flight: the fold is pure latency) and combine through LDS.
-constexpr int kFoldBlock = 1024;
-constexpr int kFoldSlices = kFoldBlock / kRowsPerBlock;
+// dst[r] (+)= sum over chunks of partial[c][r], for up to two partial arrays:
+// slice s of a block's 64 takes the chunks s, s + 64, ...; the slices combine
+// through LDS in index order.
 template <typename T>
 __device__ __forceinline__ void fold_rows_block(int block, int rows, int chunks, const float* __restrict__ part_a,
                                                 const float* __restrict__ part_b, typename T::storage* dst_a,
                                                 typename T::storage* dst_b, int accumulate,
-                                                float (*red)[kFoldSlices][kRowsPerBlock]) {
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-  const int r = block * kRowsPerBlock + tx;
+                                                float (*red)[kFoldSlices][kFoldRows]) {
+  const int tx = threadIdx.x % kFoldRows, ty = threadIdx.x / kFoldRows;
+  const int r = block * kFoldRows + tx;
   float sa = 0.f, sb = 0.f;
   if (r < rows) {
 #pragma unroll 4
@@ -121,7 +124,7 @@ __global__ __launch_bounds__(kFoldBlock) void fold_rows_kernel(int rows, int chu
                                                                const float* __restrict__ part_b,
                                                                typename T::storage* dst_a, typename T::storage* dst_b,
                                                                int accumulate) {
-  __shared__ float red[2][kFoldSlices][kRowsPerBlock];
+  __shared__ float red[2][kFoldSlices][kFoldRows];
   fold_rows_block<T>(blockIdx.x, rows, chunks, part_a, part_b, dst_a, dst_b, accumulate, red);
 }
 

@@ -19,7 +19,12 @@ template <typename T, int V>
 __global__ __launch_bounds__(kBlock) void layernorm_fwd_kernel(int rows, int cols,
                                                                const typename T::storage* x, float eps,
                                                                typename T::storage* y,  // may be x (in place)
-                                                               float* __restrict__ std_out) {
+                                                               float* __restrict__ std_out,
+                                                               // optional second result z = y * (gamma + mb) + beta,
+                                                               // gamma / beta one value per row (from y as stored)
+                                                               const typename T::storage* __restrict__ gamma,
+                                                               const typename T::storage* __restrict__ beta, float mb,
+                                                               typename T::storage* __restrict__ z) {
   const int lane = threadIdx.x & 63;
   const int wave = blockIdx.x * kWaves + (threadIdx.x >> 6);
   const int nwaves = gridDim.x * kWaves;
@@ -49,6 +54,14 @@ __global__ __launch_bounds__(kBlock) void layernorm_fwd_kernel(int rows, int col
 #pragma unroll
       for (int e = 0; e < V; ++e) v[e] = (v[e] - mean) * inv;
       st<T, V>(y + base + r, v);
+      if (z) {
+        float gv[V], bv[V];
+        ld<T, V>(gamma + r, gv);
+        ld<T, V>(beta + r, bv);
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[e] = to_float<T>(from_float<T>(v[e])) * (gv[e] + mb) + bv[e];
+        st<T, V>(z + base + r, v);
+      }
     }
     if (lane == 0) std_out[c] = sd;
   }
@@ -98,6 +111,103 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_kernel(int rows, int col
   }
 }
 
+// Backward of z = LayerNorm(x) * (gamma + mb) + beta in one pass over dz: the
+// gradient of the normalised values da = dz * (gamma + mb) (rounded to the
+// storage type, as the separate CwiseProdAdd backward stores it) is formed on
+// the fly and pushed through the LayerNorm formula above into dx; the row sums
+// dgamma += sum_c dz (*) y and dbeta += sum_c dz stay in registers over the
+// columns of a wave and leave as one fp32 partial row per workgroup.  One wave
+// per column, rows <= 64 * V * ITERS (ITERS vectors per lane; at most kLnRowIters).
+constexpr int kLnRowIters = 4;
+template <typename T, int V, int ITERS>
+__global__ __launch_bounds__(kBlock) void layernorm_affine_bwd_kernel(
+    int rows, int cols, const typename T::storage* __restrict__ dz, const typename T::storage* __restrict__ y,
+    const float* __restrict__ std_in, const typename T::storage* __restrict__ gamma, float mb,
+    typename T::storage* dx, int accumulate, float* __restrict__ part_g, float* __restrict__ part_b) {
+  __shared__ float red[kWaves][64 * V];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int wave = blockIdx.x * kWaves + w;
+  const int nwaves = gridDim.x * kWaves;
+  const float inv_rows = 1.f / static_cast<float>(rows);
+  float scale[ITERS][V], sg[ITERS][V], sb[ITERS][V];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int r = (it * 64 + lane) * V;
+#pragma unroll
+    for (int e = 0; e < V; ++e) scale[it][e] = sg[it][e] = sb[it][e] = 0.f;
+    if (r < rows) {
+      ld<T, V>(gamma + r, scale[it]);
+#pragma unroll
+      for (int e = 0; e < V; ++e) scale[it][e] += mb;
+    }
+  }
+  for (int c = wave; c < cols; c += nwaves) {
+    const size_t base = static_cast<size_t>(c) * rows;
+    float g[ITERS][V], yv[ITERS][V];
+    float s = 0.f, d = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int r = (it * 64 + lane) * V;
+#pragma unroll
+      for (int e = 0; e < V; ++e) g[it][e] = yv[it][e] = 0.f;
+      if (r < rows) {
+        ld<T, V>(dz + base + r, g[it]);
+        ld<T, V>(y + base + r, yv[it]);
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          sg[it][e] += g[it][e] * yv[it][e];
+          sb[it][e] += g[it][e];
+          g[it][e] = to_float<T>(from_float<T>(g[it][e] * scale[it][e]));  // da as the separate kernel stores it
+          s += g[it][e];
+          d += g[it][e] * yv[it][e];
+        }
+      }
+    }
+    if (dx) {
+      const float gmean = wave_sum(s) * inv_rows;
+      const float dot = wave_sum(d) * inv_rows;
+      const float inv = 1.f / std_in[c];
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int r = (it * 64 + lane) * V;
+        if (r < rows) {
+          float old[V];
+#pragma unroll
+          for (int e = 0; e < V; ++e) old[e] = 0.f;
+          if (accumulate) ld<T, V>(dx + base + r, old);
+#pragma unroll
+          for (int e = 0; e < V; ++e) old[e] += (g[it][e] - gmean - yv[it][e] * dot) * inv;
+          st<T, V>(dx + base + r, old);
+        }
+      }
+    }
+  }
+  if (!part_g) return;
+  // The four waves' row sums -> one partial row per workgroup (waves 1..3 hand theirs to wave 0).
+#pragma unroll
+  for (int which = 0; which < 2; ++which) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int r = (it * 64 + lane) * V;
+      float (&mine)[V] = which ? sb[it] : sg[it];
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < V; ++e) red[w][lane * V + e] = mine[e];
+      __syncthreads();
+      if (w == 0 && r < rows) {
+        float* out = (which ? part_b : part_g) + static_cast<size_t>(blockIdx.x) * rows + r;
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          float t = 0.f;
+#pragma unroll
+          for (int k = 0; k < kWaves; ++k) t += red[k][lane * V + e];
+          out[e] = t;
+        }
+      }
+    }
+  }
+}
+
 // y = a * (b + mb) + c; with `broadcast`, b and c are [rows] vectors applied
 // to every column (rows is a multiple of V then).
 template <typename T, int V>
@@ -128,11 +238,11 @@ __global__ __launch_bounds__(kBlock) void cwise_prod_add_bwd_flat_kernel(size_t 
                                                                          const typename T::storage* __restrict__ b,
                                                                          float mb, typename T::storage* da,
                                                                          typename T::storage* db,
-                                                                         typename T::storage* dc) {
+                                                                         typename T::storage* dc, int add_da) {
   for (size_t i = blockIdx.x * static_cast<size_t>(kBlock) + threadIdx.x; i < n;
        i += static_cast<size_t>(gridDim.x) * kBlock) {
     const float g = to_float<T>(dy[i]);
-    if (da) da[i] = from_float<T>(to_float<T>(da[i]) + g * (to_float<T>(b[i]) + mb));
+    if (da) da[i] = from_float<T>((add_da ? to_float<T>(da[i]) : 0.f) + g * (to_float<T>(b[i]) + mb));
     if (db) db[i] = from_float<T>(to_float<T>(db[i]) + g * to_float<T>(a[i]));
     if (dc) dc[i] = from_float<T>(to_float<T>(dc[i]) + g);
   }
@@ -144,7 +254,7 @@ template <typename T, int V>
 __global__ __launch_bounds__(rowred::kBlock) void cwise_prod_add_bwd_bcast_kernel(
     int nrows, int cols, int cols_per_chunk, const typename T::storage* __restrict__ dy,
     const typename T::storage* __restrict__ a, const typename T::storage* __restrict__ b, float mb,
-    typename T::storage* da, float* __restrict__ part_b, float* __restrict__ part_c) {
+    typename T::storage* da, float* __restrict__ part_b, float* __restrict__ part_c, int add_da) {
   __shared__ float red[rowred::kSlices * V * 64];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int r = (blockIdx.x * rowred::kRowsPerBlock + tx) * V;
@@ -174,7 +284,7 @@ __global__ __launch_bounds__(rowred::kBlock) void cwise_prod_add_bwd_bcast_kerne
           const size_t i = static_cast<size_t>(cu) * nrows + r;
           ld<T, V>(dy + i, g[u]);
           ld<T, V>(a + i, av[u]);
-          if (da) ld<T, V>(da + i, d[u]);
+          if (da && add_da) ld<T, V>(da + i, d[u]);
         }
       }
 #pragma unroll
@@ -409,8 +519,90 @@ int ginn_hip_layernorm_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, in
   const unsigned grid = grid_for(static_cast<size_t>(cols), kWaves, ctx->num_cus);
   const bool vec = vec8_ok({x, y}, {static_cast<size_t>(rows)});
   GH_DISPATCH_DTYPE_V(dtype, vec, (layernorm_fwd_kernel<T, V><<<grid, kBlock, 0, ctx->stream>>>(
-      rows, cols, static_cast<const T::storage*>(x), eps, static_cast<T::storage*>(y), std_out)));
+      rows, cols, static_cast<const T::storage*>(x), eps, static_cast<T::storage*>(y), std_out, nullptr, nullptr, 0.f,
+      nullptr)));
   GH_HIP(hipGetLastError());
+  return kOk;
+}
+
+int ginn_hip_layernorm_affine_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* x, float eps,
+                                  const void* gamma, const void* beta, float multiplier_bias, void* y, float* std_out,
+                                  void* z) {
+  GH_CHECK_ARG(ctx, "ginn_hip_layernorm_affine_fwd: ctx is NULL");
+  GH_CHECK_ARG(rows >= 0 && cols >= 0, "ginn_hip_layernorm_affine_fwd: negative dimension");
+  if (rows == 0 || cols == 0) return kOk;
+  GH_CHECK_ARG(x && gamma && beta && y && std_out && z, "ginn_hip_layernorm_affine_fwd: NULL pointer");
+  GH_CHECK_ARG(z != x && z != y, "ginn_hip_layernorm_affine_fwd: z must be an array of its own");
+  GH_HIP(hipSetDevice(ctx->device));
+  const unsigned grid = grid_for(static_cast<size_t>(cols), kWaves, ctx->num_cus);
+  const bool vec = vec8_ok({x, y, z, gamma, beta}, {static_cast<size_t>(rows)});
+  GH_DISPATCH_DTYPE_V(dtype, vec, (layernorm_fwd_kernel<T, V><<<grid, kBlock, 0, ctx->stream>>>(
+      rows, cols, static_cast<const T::storage*>(x), eps, static_cast<T::storage*>(y), std_out,
+      static_cast<const T::storage*>(gamma), static_cast<const T::storage*>(beta), multiplier_bias,
+      static_cast<T::storage*>(z))));
+  GH_HIP(hipGetLastError());
+  return kOk;
+}
+
+int ginn_hip_layernorm_affine_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* dz,
+                                  const void* y, const float* std_in, const void* gamma, float multiplier_bias,
+                                  void* dx, int accumulate, void* dgamma, void* dbeta) {
+  GH_CHECK_ARG(ctx, "ginn_hip_layernorm_affine_bwd: ctx is NULL");
+  GH_CHECK_ARG(rows >= 0 && cols >= 0, "ginn_hip_layernorm_affine_bwd: negative dimension");
+  if (rows == 0 || cols == 0 || (!dx && !dgamma && !dbeta)) return kOk;
+  GH_CHECK_ARG(dz && y && std_in && gamma, "ginn_hip_layernorm_affine_bwd: NULL pointer");
+  GH_CHECK_ARG((dgamma == nullptr) == (dbeta == nullptr),
+               "ginn_hip_layernorm_affine_bwd: dgamma and dbeta come together");
+  GH_CHECK_ARG(dx != dz && dx != y, "ginn_hip_layernorm_affine_bwd: dx must not be an input");
+  GH_HIP(hipSetDevice(ctx->device));
+  const bool vec = vec8_ok({dz, y, dx, gamma}, {static_cast<size_t>(rows)});
+  const int per_iter = 64 * (vec ? 8 : 1);
+  if (rows > per_iter * kLnRowIters) {
+    // A column longer than a wave holds in registers: the two steps one after the other, through a
+    // temporary for the gradient of the normalised values.
+    void* da = nullptr;
+    const size_t bytes = static_cast<size_t>(rows) * cols * dtype_size(dtype);
+    if (int rc = ginn_hip_malloc(ctx, bytes, &da)) return rc;
+    int rc = ginn_hip_memset(ctx, da, 0, bytes);
+    if (rc == kOk)
+      rc = ginn_hip_cwise_prod_add_bwd(ctx, dtype, rows, cols, dz, y, gamma, multiplier_bias, 1, da, dgamma, dbeta);
+    if (rc == kOk && dx)
+      rc = (accumulate ? ginn_hip_layernorm_bwd : ginn_hip_layernorm_bwd_assign)(ctx, dtype, rows, cols, da, y,
+                                                                                  std_in, dx);
+    const int rc_free = ginn_hip_free(ctx, da);
+    return rc != kOk ? rc : rc_free;
+  }
+  std::lock_guard<std::mutex> lock(ctx->mutex);
+  // At most 2 workgroups per CU: every workgroup leaves a partial row for the fold.
+  unsigned grid = grid_for(static_cast<size_t>(cols), kWaves, ctx->num_cus);
+  const unsigned cap = static_cast<unsigned>(2 * ctx->num_cus);
+  if (grid > cap) grid = cap;
+  const size_t part_bytes = static_cast<size_t>(grid) * rows * sizeof(float);
+  rowred::Partials room{nullptr, false};
+  if (dgamma) {
+    GH_CHECK_ARG(2 * part_bytes <= ctx->workspace_bytes, "ginn_hip_layernorm_affine_bwd: workspace too small for %d rows",
+                 rows);
+    room = rowred::take_partials(ctx, 2 * part_bytes);
+  }
+  float* part_g = room.base;
+  float* part_b = part_g ? part_g + static_cast<size_t>(grid) * rows : nullptr;
+  const int iters = (rows + per_iter - 1) / per_iter;
+#define GH_LN_BWD(ITERS)                                                                                       \
+  GH_DISPATCH_DTYPE_V(dtype, vec, (layernorm_affine_bwd_kernel<T, V, ITERS><<<grid, kBlock, 0, ctx->stream>>>( \
+      rows, cols, static_cast<const T::storage*>(dz), static_cast<const T::storage*>(y), std_in,              \
+      static_cast<const T::storage*>(gamma), multiplier_bias, static_cast<T::storage*>(dx), accumulate,       \
+      part_g, part_b)))
+  if (iters <= 1) {
+    GH_LN_BWD(1);
+  } else if (iters == 2) {
+    GH_LN_BWD(2);
+  } else {
+    GH_LN_BWD(kLnRowIters);
+  }
+#undef GH_LN_BWD
+  GH_HIP(hipGetLastError());
+  if (dgamma)
+    return rowred::finish(ctx, {dtype, rows, static_cast<int>(grid), 1, part_g, part_b, dgamma, dbeta}, room.deferred);
   return kOk;
 }
 
@@ -457,37 +649,52 @@ int ginn_hip_cwise_prod_add_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int row
   return kOk;
 }
 
-int ginn_hip_cwise_prod_add_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* dy,
-                                const void* a, const void* b, float multiplier_bias, int broadcast, void* da,
-                                void* db, void* dc) {
-  GH_CHECK_ARG(ctx, "ginn_hip_cwise_prod_add_bwd: ctx is NULL");
-  GH_CHECK_ARG(rows >= 0 && cols >= 0, "ginn_hip_cwise_prod_add_bwd: negative dimension");
+static int cwise_prod_add_bwd(const char* who, ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols,
+                              const void* dy, const void* a, const void* b, float multiplier_bias, int broadcast,
+                              void* da, void* db, void* dc, int add_da) {
+  GH_CHECK_ARG(ctx, "%s: ctx is NULL", who);
+  GH_CHECK_ARG(rows >= 0 && cols >= 0, "%s: negative dimension", who);
   if (rows == 0 || cols == 0 || (!da && !db && !dc)) return kOk;
-  GH_CHECK_ARG(dy && a && b, "ginn_hip_cwise_prod_add_bwd: NULL pointer");
+  GH_CHECK_ARG(dy && a && b, "%s: NULL pointer", who);
   GH_HIP(hipSetDevice(ctx->device));
   if (!broadcast) {
     const size_t n = static_cast<size_t>(rows) * cols;
     const unsigned grid = grid_for(n, kBlock, ctx->num_cus);
     GH_DISPATCH_DTYPE(dtype, (cwise_prod_add_bwd_flat_kernel<T><<<grid, kBlock, 0, ctx->stream>>>(
         n, static_cast<const T::storage*>(dy), static_cast<const T::storage*>(a), static_cast<const T::storage*>(b),
-        multiplier_bias, static_cast<T::storage*>(da), static_cast<T::storage*>(db), static_cast<T::storage*>(dc))));
+        multiplier_bias, static_cast<T::storage*>(da), static_cast<T::storage*>(db), static_cast<T::storage*>(dc),
+        add_da)));
     GH_HIP(hipGetLastError());
     return kOk;
   }
   std::lock_guard<std::mutex> lock(ctx->mutex);  // the workspace holds the partials
   const bool vec = vec8_ok({dy, a, b, da}, {static_cast<size_t>(rows)});
   const rowred::Plan plan = rowred::plan(rows, cols, ctx->num_cus, ctx->workspace_bytes, 2, vec ? 8 : 1);
-  GH_CHECK_ARG(plan.chunks >= 1, "ginn_hip_cwise_prod_add_bwd: workspace too small for %d rows", rows);
+  GH_CHECK_ARG(plan.chunks >= 1, "%s: workspace too small for %d rows", who, rows);
   const rowred::Partials room = rowred::take_partials(ctx, 2 * static_cast<size_t>(plan.chunks) * rows * sizeof(float));
   float* part_b = room.base;
   float* part_c = part_b + static_cast<size_t>(plan.chunks) * rows;
   GH_DISPATCH_DTYPE_V(dtype, vec, (cwise_prod_add_bwd_bcast_kernel<T, V><<<dim3(plan.row_blocks, plan.chunks),
                                                                            rowred::kBlock, 0, ctx->stream>>>(
       rows, cols, plan.cols_per_chunk, static_cast<const T::storage*>(dy), static_cast<const T::storage*>(a),
-      static_cast<const T::storage*>(b), multiplier_bias, static_cast<T::storage*>(da), part_b, part_c)));
+      static_cast<const T::storage*>(b), multiplier_bias, static_cast<T::storage*>(da), part_b, part_c, add_da)));
   GH_HIP(hipGetLastError());
   if (db || dc) return rowred::finish(ctx, {dtype, rows, plan.chunks, 1, part_b, part_c, db, dc}, room.deferred);
   return kOk;
+}
+
+int ginn_hip_cwise_prod_add_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* dy,
+                                const void* a, const void* b, float multiplier_bias, int broadcast, void* da,
+                                void* db, void* dc) {
+  return cwise_prod_add_bwd("ginn_hip_cwise_prod_add_bwd", ctx, dtype, rows, cols, dy, a, b, multiplier_bias, broadcast,
+                            da, db, dc, 1);
+}
+
+int ginn_hip_cwise_prod_add_bwd_assign(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows, int cols, const void* dy,
+                                       const void* a, const void* b, float multiplier_bias, int broadcast, void* da,
+                                       void* db, void* dc) {
+  return cwise_prod_add_bwd("ginn_hip_cwise_prod_add_bwd_assign", ctx, dtype, rows, cols, dy, a, b, multiplier_bias,
+                            broadcast, da, db, dc, 0);
 }
 
 int ginn_hip_permute(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rank, const long long* host_dims,

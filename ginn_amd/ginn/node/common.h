@@ -5,6 +5,7 @@
 #define GINN_NODE_COMMON_H
 
 #include <ginn/node/data.h>
+#include <ginn/node/layernorm.h>
 #include <ginn/nonlin.h>
 
 namespace ginn {
@@ -218,7 +219,8 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
 
   void forward_() override {
     internal::require_gpu(this->dev(), "CwiseProdAdd");
-    const Shape s0 = a_->value().shape(), s1 = b_->value().shape(), s2 = c_->value().shape();
+    // shape(), not value(): a LayerNorm in front that has not run yet stays so
+    const Shape s0 = a_->shape(), s1 = b_->value().shape(), s2 = c_->value().shape();
     if (s0 == s1 && s1 == s2) {
       broadcast_ = false;
     } else if (s1.size() == 1 && s2.size() == 1) {
@@ -228,6 +230,17 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
       GINN_THROW("Unexpected shapes for CwiseProdAdd!");
     }
     value().resize(s0);
+    // Right behind a LayerNorm whose kernel has not run yet: normalisation and
+    // the gamma / beta step as one pass (same values).
+    if (LayerNormNode<Scalar>* ln = broadcast_ ? layer_norm() : nullptr; ln && ln->pending_) {
+      ln->pending_ = false;
+      auto& x = ln->in_->value();
+      GINN_HIP_CALL(ginn_hip_layernorm_affine_fwd(
+          internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()), static_cast<int>(x.cols()), x.data(),
+          ln->eps_, b_->value().data(), c_->value().data(), multiplier_bias_, ln->raw_value().data(), ln->std_.data(),
+          value().data()));
+      return;
+    }
     auto& a = a_->value();
     GINN_HIP_CALL(ginn_hip_cwise_prod_add_fwd(internal::ctx_of(a), dtype_of<Scalar>(), static_cast<int>(a.rows()),
                                               static_cast<int>(a.cols()), a.data(), b_->value().data(),
@@ -237,11 +250,32 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
   void backward_() override {
     auto& a = a_->value();
     internal::PostponeFolds later(internal::ctx_of(a), *b_, *c_);  // scale / shift gradients: complete at the pass's end
-    GINN_HIP_CALL(ginn_hip_cwise_prod_add_bwd(
+    // A flagged gradient of a means: this node is its only user and overwrites.
+    const bool fresh = a_->has_grad() && a_->take_lazy_zero();
+    LayerNormNode<Scalar>* ln = fresh && broadcast_ && b_->has_grad() == c_->has_grad() ? layer_norm() : nullptr;
+    if (ln) {
+      // ... and behind a LayerNorm nobody else will read that gradient either: both
+      // backward steps as one pass, the LayerNorm node skips its own.
+      auto& x = ln->in_;
+      const bool x_fresh = x->has_grad() && x->take_lazy_zero();
+      GINN_HIP_CALL(ginn_hip_layernorm_affine_bwd(
+          internal::ctx_of(a), dtype_of<Scalar>(), static_cast<int>(a.rows()), static_cast<int>(a.cols()),
+          grad().data(), a.data(), ln->std_.data(), b_->value().data(), multiplier_bias_,
+          x->has_grad() ? x->grad().data() : nullptr, x_fresh ? 0 : 1, b_->has_grad() ? b_->grad().data() : nullptr,
+          c_->has_grad() ? c_->grad().data() : nullptr));
+      ln->skip_backward_ = true;
+      return;
+    }
+    GINN_HIP_CALL((fresh ? ginn_hip_cwise_prod_add_bwd_assign : ginn_hip_cwise_prod_add_bwd)(
         internal::ctx_of(a), dtype_of<Scalar>(), static_cast<int>(a.rows()), static_cast<int>(a.cols()),
         grad().data(), a.data(), b_->value().data(), multiplier_bias_, broadcast_ ? 1 : 0,
         a_->has_grad() ? a_->grad().data() : nullptr, b_->has_grad() ? b_->grad().data() : nullptr,
         c_->has_grad() ? c_->grad().data() : nullptr));
+  }
+  // The LayerNorm this node follows directly, if any (not one that normalises in place).
+  LayerNormNode<Scalar>* layer_norm() const {
+    auto* ln = dynamic_cast<LayerNormNode<Scalar>*>(a_.get());
+    return ln && ln->may_postpone() ? ln : nullptr;
   }
 
  public:
@@ -252,6 +286,10 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
                    Bias multiplier_bias = Bias(0))
       : BaseDataNode<Scalar>({a, b, c}), a_(a), b_(b), c_(c),
         multiplier_bias_(static_cast<float>(multiplier_bias)) {}
+  // The gradient of a is overwritten when it holds no value yet; b and c are added to.
+  BaseNode::GradUse grad_use(size_t index) const override {
+    return index == 0 ? BaseNode::GradUse::Overwrites : BaseNode::GradUse::Accumulates;
+  }
   std::string name() const override { return "CwiseProdAdd"; }
 };
 GINN_MAKE_SCALAR_FORWARDING_FACTORY(CwiseProdAdd);

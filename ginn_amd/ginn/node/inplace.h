@@ -258,6 +258,7 @@ class InPlaceLayerNormNode : public LayerNormNode<Scalar> {
  public:
   using LayerNormNode<Scalar>::LayerNormNode;
   GINN_INPLACE_ALIASES(in_)
+  bool may_postpone() const override { return false; }
   std::string name() const override { return "InPlaceLayerNorm"; }
 };
 GINN_MAKE_SCALAR_FORWARDING_FACTORY(InPlaceLayerNorm);

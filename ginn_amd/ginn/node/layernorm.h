@@ -11,21 +11,52 @@
 namespace ginn {
 
 template <typename Scalar>
+class CwiseProdAddNode;
+
+// The normalisation is postponed until the value is read: a CwiseProdAdd right
+// behind it (the gamma / beta step, examples/min-gpt.cu.cpp:100-103) then runs
+// both as one pass (ginn_hip_layernorm_affine_fwd), and, when this node's
+// gradient has no other user, both backward steps as one
+// (ginn_hip_layernorm_affine_bwd).  Any other reader gets the value as usual.
+template <typename Scalar>
 class LayerNormNode : public BaseDataNode<Scalar> {
+  friend class CwiseProdAddNode<Scalar>;
+
  protected:
   NodePtr<Scalar> in_;
   float eps_;
   Tensor<float> std_;
+  mutable bool pending_ = false;  // forward() has run, the kernel has not
+  bool skip_backward_ = false;    // the node behind has done this node's backward as well
 
-  void forward_() override {
-    internal::require_gpu(this->dev(), "LayerNorm");
+  // Nodes that normalise in place run at once.
+  virtual bool may_postpone() const { return true; }
+  Tensor<Scalar>& raw_value() const { return const_cast<Tensor<Scalar>&>(BaseDataNode<Scalar>::value()); }
+  void normalise() const {
     auto& x = in_->value();
-    value().resize(x.shape());
-    std_.resize({1, x.cols()});
+    Tensor<Scalar>& y = may_postpone() ? raw_value() : const_cast<LayerNormNode*>(this)->value();
     GINN_HIP_CALL(ginn_hip_layernorm_fwd(internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()),
-                                         static_cast<int>(x.cols()), x.data(), eps_, value().data(), std_.data()));
+                                         static_cast<int>(x.cols()), x.data(), eps_, y.data(),
+                                         const_cast<Tensor<float>&>(std_).data()));
+  }
+  void forward_() override {
+    internal::require_gpu(in_->dev(), "LayerNorm");
+    const Shape s = in_->shape();
+    const Size rows = s.empty() ? 1 : s[0];
+    std_.resize({1, rows > 0 ? Tensor<Scalar>::size(s) / rows : 0});
+    if (may_postpone()) {
+      raw_value().resize(s);
+      pending_ = true;
+    } else {
+      value().resize(s);
+      normalise();
+    }
   }
   void backward_() override {
+    if (skip_backward_) {
+      skip_backward_ = false;
+      return;
+    }
     if (!in_->has_grad()) return;
     auto& y = value();
     const bool fresh = in_->take_lazy_zero();
@@ -35,8 +66,17 @@ class LayerNormNode : public BaseDataNode<Scalar> {
   }
 
  public:
-  using BaseDataNode<Scalar>::value;
+  const Tensor<Scalar>& value() const override {
+    if (pending_) {
+      pending_ = false;
+      normalise();
+    }
+    return BaseDataNode<Scalar>::value();
+  }
+  using Node<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
+  Shape shape() const override { return pending_ ? in_->shape() : value().shape(); }
+  DevPtr dev() const override { return in_->dev(); }
   BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; }
   LayerNormNode(const NodePtr<Scalar>& in, double eps = 1e-8)
       : BaseDataNode<Scalar>({in}), in_(in), eps_(static_cast<float>(eps)), std_(in->dev()) {}

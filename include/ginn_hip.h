@@ -434,6 +434,42 @@ int ginn_hip_cwise_prod_add_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
                                 const void* a, const void* b,
                                 float multiplier_bias, int broadcast, void* da,
                                 void* db, void* dc);
+/* The same with da assigned instead of added to (a gradient that reset_grad()
+ * had just zeroed, ginn/node.h:218-222); db and dc are added to as above. */
+int ginn_hip_cwise_prod_add_bwd_assign(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                                       int rows, int cols, const void* dy,
+                                       const void* a, const void* b,
+                                       float multiplier_bias, int broadcast,
+                                       void* da, void* db, void* dc);
+
+/* LayerNorm followed by the gamma / beta step, z = LayerNorm(x) * (gamma +
+ * multiplier_bias) + beta with gamma, beta [rows] vectors: the pair
+ * LayerNormNode (ginn/node/layernorm.h:31-47) + CwiseProdAddNode
+ * (ginn/node/common.h:251-296) of examples/min-gpt.cu.cpp:100-103 as one pass.
+ * y [rows x cols] receives the normalised values and std_out [cols] the
+ * statistics, as ginn_hip_layernorm_fwd leaves them (both are needed for the
+ * backward pass); z is computed from y as stored.  Same bits as the two
+ * separate calls. */
+int ginn_hip_layernorm_affine_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                                  int rows, int cols, const void* x, float eps,
+                                  const void* gamma, const void* beta,
+                                  float multiplier_bias, void* y,
+                                  float* std_out, void* z);
+/* Backward of the pair for a gradient of y that holds no value yet (y has no
+ * other user): dx (+)= LayerNorm backward of da = dz * (gamma +
+ * multiplier_bias), da rounded to the storage type but never stored;
+ * dgamma += sum_c dz (*) y, dbeta += sum_c dz (both or neither; their fold can
+ * be postponed, see ginn_hip_defer_folds).  dx may be NULL; accumulate == 0
+ * assigns dx.  Results as from ginn_hip_cwise_prod_add_bwd_assign followed by
+ * ginn_hip_layernorm_bwd(_assign) up to fp32 rounding (the compiler contracts
+ * the same expressions differently in the two kernels; the row sums are taken
+ * in another order of the columns). */
+int ginn_hip_layernorm_affine_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                                  int rows, int cols, const void* dz,
+                                  const void* y, const float* std_in,
+                                  const void* gamma, float multiplier_bias,
+                                  void* dx, int accumulate, void* dgamma,
+                                  void* dbeta);
 
 /* PermuteNode (ginn/node/layout.h:723-821): dst has extents
  * dims[perm[0]], dims[perm[1]], ... and dst[i_perm] = src[i] (Eigen's

@@ -71,6 +71,80 @@ def test_layernorm(dev, dt, rows, cols):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(768, 520), (64, 5), (8, 3), (1536, 33), (2048, 70), (520, 1030), (12, 7),
+                                       (2056, 9), (300, 5)])
+@pytest.mark.parametrize("accumulate", [0, 1])
+def test_layernorm_affine_as_one_pass(dev, dt, rows, cols, accumulate):
+    """ginn_hip_layernorm_affine_fwd / _bwd against ginn_hip_layernorm_fwd + ginn_hip_cwise_prod_add_fwd and
+    ginn_hip_cwise_prod_add_bwd_assign + ginn_hip_layernorm_bwd(_assign): normalised values, statistics and z
+    bit for bit; dx and the gamma / beta gradients (row sums taken in another order of the columns) within fp32
+    rounding; and all of it against numpy.  Columns of 1, 2 and 4 vectors per lane, columns that
+    are not multiples of 8 (scalar accesses) and ones too long for the registers (the two steps inside)."""
+    from gpu_util import TOL, round_to
+    rng = np.random.default_rng(rows * 7 + cols)
+    x = round_to(rng.standard_normal((rows, cols)) * 2 + 0.5, dt)
+    gamma = round_to(rng.standard_normal(rows) * 0.3, dt)
+    beta = round_to(rng.standard_normal(rows), dt)
+    dz = round_to(rng.standard_normal((rows, cols)), dt)
+    old_dx = round_to(rng.standard_normal((rows, cols)), dt)
+    old_dg = round_to(rng.standard_normal(rows), dt)
+    old_db = round_to(rng.standard_normal(rows), dt)
+    mb, eps = 1.0, 1e-8
+    t = dev.torch
+    put = lambda a: dev.put(a, dt)
+    (bx, px, _), (bg, pg, _), (bb, pb, _), (bdz, pdz, _) = put(x), put(gamma), put(beta), put(dz)
+
+    def separate():
+        (by, py, _), (bz, pz, _), (bda, pda, _) = put(np.zeros_like(x)), put(np.zeros_like(x)), put(np.full_like(x, 3.0))
+        (bdx, pdx, _), (bdg, pdg, _), (bdb, pdb, _) = put(old_dx), put(old_dg), put(old_db)
+        std = t.zeros(cols, dtype=t.float32, device="cuda")
+        dev.lib.call("ginn_hip_layernorm_fwd", dev.ctx, dt, rows, cols, c_void_p(px), eps, c_void_p(py),
+                     c_void_p(std.data_ptr()))
+        dev.lib.call("ginn_hip_cwise_prod_add_fwd", dev.ctx, dt, rows, cols, c_void_p(py), c_void_p(pg), c_void_p(pb),
+                     mb, 1, c_void_p(pz))
+        dev.lib.call("ginn_hip_cwise_prod_add_bwd_assign", dev.ctx, dt, rows, cols, c_void_p(pdz), c_void_p(py),
+                     c_void_p(pg), mb, 1, c_void_p(pda), c_void_p(pdg), c_void_p(pdb))
+        dev.lib.call("ginn_hip_layernorm_bwd" if accumulate else "ginn_hip_layernorm_bwd_assign", dev.ctx, dt, rows,
+                     cols, c_void_p(pda), c_void_p(py), c_void_p(std.data_ptr()), c_void_p(pdx))
+        dev.sync()
+        return [dev.get(b, s) for b, s in ((by, x.shape), (bz, x.shape), (bdx, x.shape), (bdg, (rows,)),
+                                           (bdb, (rows,)))] + [std.cpu().numpy()]
+
+    def fused():
+        (by, py, _), (bz, pz, _) = put(np.zeros_like(x)), put(np.zeros_like(x))
+        (bdx, pdx, _), (bdg, pdg, _), (bdb, pdb, _) = put(old_dx), put(old_dg), put(old_db)
+        std = t.zeros(cols, dtype=t.float32, device="cuda")
+        dev.lib.call("ginn_hip_layernorm_affine_fwd", dev.ctx, dt, rows, cols, c_void_p(px), eps, c_void_p(pg),
+                     c_void_p(pb), mb, c_void_p(py), c_void_p(std.data_ptr()), c_void_p(pz))
+        dev.lib.call("ginn_hip_layernorm_affine_bwd", dev.ctx, dt, rows, cols, c_void_p(pdz), c_void_p(py),
+                     c_void_p(std.data_ptr()), c_void_p(pg), mb, c_void_p(pdx), accumulate, c_void_p(pdg),
+                     c_void_p(pdb))
+        dev.sync()
+        return [dev.get(b, s) for b, s in ((by, x.shape), (bz, x.shape), (bdx, x.shape), (bdg, (rows,)),
+                                           (bdb, (rows,)))] + [std.cpu().numpy()]
+
+    y1, z1, dx1, dg1, db1, std1 = separate()
+    y2, z2, dx2, dg2, db2, std2 = fused()
+    np.testing.assert_array_equal(y2, y1)
+    np.testing.assert_array_equal(std2, std1)
+    np.testing.assert_array_equal(z2, z1)
+    assert rel_fro(dx2, dx1) <= {capi.F32: 1e-6}.get(dt, TOL[dt] / 8)
+    # row sums over `cols` terms in fp32, rounded to the storage type once
+    assert rel_fro(dg2, dg1) <= {capi.F32: 2e-6}.get(dt, TOL[dt] / 4)
+    assert rel_fro(db2, db1) <= {capi.F32: 2e-6}.get(dt, TOL[dt] / 4)
+    # against numpy, from the values the device stored
+    y64 = y2.astype(np.float64)
+    want_z = y64 * (gamma.astype(np.float64)[:, None] + mb) + beta.astype(np.float64)[:, None]
+    assert rel_fro(z2, want_z) <= TOL[dt]
+    da = round_to(dz.astype(np.float64) * (gamma.astype(np.float64)[:, None] + mb), dt).astype(np.float64)
+    want_dx = (old_dx if accumulate else 0) + N.layernorm_backward(da, y64, std2.astype(np.float64))
+    if rows > 1:
+        assert rel_fro(dx2, want_dx) <= TOL[dt] * 2
+    assert rel_fro(dg2, old_dg + (dz.astype(np.float64) * y64).sum(axis=1)) <= TOL[dt]
+    assert rel_fro(db2, old_db + dz.astype(np.float64).sum(axis=1)) <= TOL[dt]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("rows,cols,broadcast", [(768, 40, 1), (5, 3, 1), (5, 3, 0), (300, 257, 1), (1, 9, 1)])
 def test_cwise_prod_add(dev, dt, rows, cols, broadcast):
     from gpu_util import TOL, round_to
