@@ -573,9 +573,9 @@ int ginn_hip_layernorm_affine_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int r
     return rc != kOk ? rc : rc_free;
   }
   std::lock_guard<std::mutex> lock(ctx->mutex);
-  // At most 2 workgroups per CU: every workgroup leaves a partial row for the fold.
+  // At most one workgroup per CU: every workgroup leaves a partial row for the fold.
   unsigned grid = grid_for(static_cast<size_t>(cols), kWaves, ctx->num_cus);
-  const unsigned cap = static_cast<unsigned>(2 * ctx->num_cus);
+  const unsigned cap = static_cast<unsigned>(ctx->num_cus);
   if (grid > cap) grid = cap;
   const size_t part_bytes = static_cast<size_t>(grid) * rows * sizeof(float);
   rowred::Partials room{nullptr, false};
