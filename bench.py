@@ -574,6 +574,13 @@ def main():
             "kernel_ms": round(kernel_ms, 4),
         },
     }
+    # A shape with fewer flops per algorithmic byte than the part has per byte of HBM bandwidth (narrow
+    # right-hand sides) is bound by memory: its roofline is algorithmic bytes per second against 8 TB/s.
+    algo_bytes = ESIZE[a.dtype] * (m * k + k * n + m * n * (2 if a.beta != 0 else 1))
+    if flops / algo_bytes < PEAK_TFLOPS[a.dtype] * 1e12 / (PEAK_HBM_GBS * 1e9):
+        gbs = algo_bytes / (kernel_ms * 1e-3) / 1e9
+        line["roofline"].update({"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                 "frac": round(gbs / PEAK_HBM_GBS, 4)})
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(m, k, min(a.cpu_panel, n), a.dtype)
     if not a.no_configs:

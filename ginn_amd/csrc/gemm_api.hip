@@ -50,7 +50,14 @@ int launch_gemm(ginn_hip_ctx* ctx, const GemmArgs& a) {
     return ginn_hip_col_dot_batched(ctx, static_cast<ginn_hip_dtype>(a.dtype), a.k,
                                     a.batch, a.A, a.B, a.beta, a.C);
   }
-  int rc = launch_gemm_skinny(ctx, a);
+  // 16-bit products with a few columns: the 128 x 64 matrix-core kernel with split K reads A as fast as
+  // the vector-ALU kernel and has the arithmetic for free (fp16 4096 x n x 4096: 7.9-8.5 us for n = 1 .. 8
+  // against 8.5-15.2 us); the vector-ALU kernel keeps fp32 (whose matrix pipe is 16 x slower) and the 16-bit
+  // shapes the matrix-core kernel does not take (unaligned operands, odd extents).
+  int rc = kUnsupported;
+  if (a.dtype != GINN_HIP_F32 && a.batch == 1 && a.n <= 8) rc = launch_gemm_mid(ctx, a);
+  if (rc != kUnsupported) return rc;
+  rc = launch_gemm_skinny(ctx, a);
   if (rc != kUnsupported) return rc;
   rc = launch_gemm_fast16(ctx, a);
   if (rc != kUnsupported) return rc;
