@@ -58,6 +58,8 @@ PROTOTYPES = {
                                       POINTER(c_void_p), POINTER(c_int)]),
     "ginn_hip_gemm_gathered": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int,
                                        c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p, c_int]),
+    "ginn_hip_gemm_outer_sum": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p,
+                                        c_int, c_int]),
     "ginn_hip_col_dot_batched": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p]),
     "ginn_hip_affine_fwd": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, POINTER(c_void_p),
                                     POINTER(c_void_p), POINTER(c_int), c_void_p, c_void_p, c_void_p]),

@@ -360,6 +360,8 @@ struct GemmArgs {
   // of the output (n entries).  bcols replaces B/ldb, ccols replaces C/ldc.
   const void* const* bcols = nullptr;
   void* const* ccols = nullptr;
+  // A (op_a N only) by the bases of its k stored columns of m elements; replaces A/lda.
+  const void* const* acols = nullptr;
   // Set by the grouped entry point: whether every column base allows 16-byte
   // loads (B) and 4-element vector stores (C).
   bool cols_vec_ld = false;

@@ -14,8 +14,10 @@ int check_gemm_args(const char* who, const GemmArgs& a) {
   GH_CHECK_ARG(a.op_b == GINN_HIP_OP_N || a.op_b == GINN_HIP_OP_T, "%s: bad op_b %d", who, a.op_b);
   GH_CHECK_ARG(a.m >= 0 && a.n >= 0 && a.k >= 0, "%s: negative dimension (m=%d n=%d k=%d)", who, a.m, a.n, a.k);
   GH_CHECK_ARG(a.batch >= 0, "%s: negative batch %d", who, a.batch);
-  const int a_rows = a.op_a == GINN_HIP_OP_N ? a.m : a.k;
-  GH_CHECK_ARG(a.lda >= (a_rows > 1 ? a_rows : 1), "%s: lda=%d smaller than the %d rows of A", who, a.lda, a_rows);
+  if (!a.acols) {
+    const int a_rows = a.op_a == GINN_HIP_OP_N ? a.m : a.k;
+    GH_CHECK_ARG(a.lda >= (a_rows > 1 ? a_rows : 1), "%s: lda=%d smaller than the %d rows of A", who, a.lda, a_rows);
+  }
   if (!a.bcols) {
     const int b_rows = a.op_b == GINN_HIP_OP_N ? a.k : a.n;
     GH_CHECK_ARG(a.ldb >= (b_rows > 1 ? b_rows : 1), "%s: ldb=%d smaller than the %d rows of B", who, a.ldb, b_rows);
@@ -25,7 +27,7 @@ int check_gemm_args(const char* who, const GemmArgs& a) {
   if (a.m == 0 || a.n == 0 || a.batch == 0) return kOk;
   GH_CHECK_ARG(a.ccols || a.C != nullptr, "%s: C is NULL", who);
   if (a.k > 0) {
-    GH_CHECK_ARG(a.A != nullptr, "%s: A is NULL", who);
+    GH_CHECK_ARG(a.acols || a.A != nullptr, "%s: A is NULL", who);
     GH_CHECK_ARG(a.bcols || a.B != nullptr, "%s: B is NULL", who);
   }
   if (a.batch > 1) {
@@ -41,7 +43,7 @@ int launch_gemm(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (a.m == 0 || a.n == 0 || a.batch == 0) return kOk;
   GH_HIP(hipSetDevice(ctx->device));
   const bool plain = a.bias == nullptr && a.pre == nullptr &&
-                     a.act == GINN_HIP_ACT_IDENTITY && a.bcols == nullptr && a.ccols == nullptr;
+                     a.act == GINN_HIP_ACT_IDENTITY && a.bcols == nullptr && a.ccols == nullptr && a.acols == nullptr;
   // Degenerate batched dot: m = n = 1 with contiguous operands.
   if (plain && a.m == 1 && a.n == 1 && a.batch > 1 && a.stride_a == a.k &&
       a.stride_b == a.k && a.stride_c == 1 &&
@@ -220,6 +222,37 @@ int ginn_hip_gemm_gathered(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
   GH_HIP(hipSetDevice(ctx->device));
   // Without a table this is an ordinary product and takes the ordinary route.
   if (!a.bcols && !a.ccols) return launch_gemm(ctx, a);
+  return launch_gemm_generic(ctx, a);
+}
+
+int ginn_hip_gemm_outer_sum(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int m, int n, int k,
+                            const void* const* dev_a_cols, const void* const* dev_b_cols, float beta, void* C,
+                            int ldc, int cols_aligned) {
+  GH_CHECK_ARG(ctx, "ginn_hip_gemm_outer_sum: ctx is NULL");
+  GH_CHECK_ARG(k == 0 || (dev_a_cols && dev_b_cols), "ginn_hip_gemm_outer_sum: NULL table");
+  GemmArgs a{};
+  a.dtype = dtype;
+  a.op_a = GINN_HIP_OP_N;
+  a.op_b = GINN_HIP_OP_T;
+  a.m = m;
+  a.n = n;
+  a.k = k;
+  a.beta = beta;
+  a.C = C;
+  a.ldc = ldc;
+  a.batch = 1;
+  if (k > 0) {
+    a.acols = dev_a_cols;
+    a.bcols = dev_b_cols;
+  } else {  // an empty sum: C <- beta * C through the ordinary route
+    a.lda = m > 1 ? m : 1;
+    a.ldb = n > 1 ? n : 1;
+  }
+  a.cols_vec_ld = cols_aligned != 0;
+  if (int rc = check_gemm_args("ginn_hip_gemm_outer_sum", a)) return rc;
+  if (m == 0 || n == 0) return kOk;
+  GH_HIP(hipSetDevice(ctx->device));
+  if (k == 0) return launch_gemm(ctx, a);
   return launch_gemm_generic(ctx, a);
 }
 

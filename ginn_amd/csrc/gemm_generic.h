@@ -46,6 +46,9 @@ struct KParams {
   // Grouped launch: B and C are given per (virtual) column, n = their count.
   const void* const* bcols;
   void* const* ccols;
+  // A given by the bases of its stored columns (only for A stored [m x k]:
+  // entry j is column j, position j along the sum).
+  const void* const* acols;
   // Split-K (batch == 1 only): blockIdx.z selects a K range of k_chunk
   // (a multiple of the K slab); the fp32 partial tile goes to
   // partial[z][col * m + row] and a second kernel folds the splits and
@@ -279,13 +282,14 @@ __global__ __launch_bounds__(kThreads) void gemm_generic_kernel(KParams p) {
   Fetch<T, BM, AKC, VECLD> fa[kDepth];
   Fetch<T, BN, BKC, VECLD> fb[kDepth];
   const S* const* bcols = reinterpret_cast<const S* const*>(p.bcols);
+  const S* const* acols = reinterpret_cast<const S* const*>(p.acols);
 
   const int ktiles = (k_end - k_begin + BK - 1) / BK;
   if (ktiles > 0) {
 #pragma unroll
     for (int j = 0; j < kDepth; ++j)
       if (j < ktiles) {
-        fa[j].load(A, p.lda, m0, k_begin + j * BK, p.m, k_end, tid);
+        fa[j].load(A, p.lda, m0, k_begin + j * BK, p.m, k_end, tid, acols);
         fb[j].load(B, p.ldb, n0, k_begin + j * BK, p.n, k_end, tid, bcols);
       }
     fa[0].store(as[0], tid);
@@ -297,7 +301,7 @@ __global__ __launch_bounds__(kThreads) void gemm_generic_kernel(KParams p) {
         const int kt = kt0 + j;
         if (kt < ktiles) {
           if (kt + kDepth < ktiles) {  // set j (slab kt) went to LDS an iteration ago
-            fa[j].load(A, p.lda, m0, k_begin + (kt + kDepth) * BK, p.m, k_end, tid);
+            fa[j].load(A, p.lda, m0, k_begin + (kt + kDepth) * BK, p.m, k_end, tid, acols);
             fb[j].load(B, p.ldb, n0, k_begin + (kt + kDepth) * BK, p.n, k_end, tid, bcols);
           }
           mma_slab<T, BM, BN, TM, TN>(as[j & 1], bs[j & 1], acc, wm, wn, lane);

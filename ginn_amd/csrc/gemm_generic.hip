@@ -29,6 +29,7 @@ int launch_dtype(ginn_hip_ctx* ctx, const GemmArgs& a) {
   p.act = a.act;
   p.bcols = a.bcols;
   p.ccols = a.ccols;
+  p.acols = a.acols;
 
   const bool akc = a.op_a == GINN_HIP_OP_T;  // A stored [k x m]: K contiguous
   const bool bkc = a.op_b == GINN_HIP_OP_N;  // B stored [k x n]: K contiguous
@@ -38,7 +39,8 @@ int launch_dtype(ginn_hip_ctx* ctx, const GemmArgs& a) {
   };
   const bool b_ok = a.bcols ? (a.cols_vec_ld && (bkc ? a.k : a.n) % VEC == 0)
                              : aligned(a.B, a.ldb, a.stride_b, bkc ? a.k : a.n);
-  const bool vec_ld = aligned(a.A, a.lda, a.stride_a, akc ? a.k : a.m) && b_ok;
+  const bool a_ok = a.acols ? (a.cols_vec_ld && a.m % VEC == 0) : aligned(a.A, a.lda, a.stride_a, akc ? a.k : a.m);
+  const bool vec_ld = a_ok && b_ok;
   const uintptr_t c_align = 4 * es;
   if (a.ccols)
     p.vec_c = a.cols_vec_c;

@@ -501,6 +501,10 @@ const char* scenario_last_error() { return g_error.c_str(); }
 // Zero fills on demand during the timed passes of the last scenario (see g_timed_fills).
 long scenario_timed_fills() { return g_timed_fills; }
 
+// Columns summed so far by products that waited for the end of their backward pass
+// (internal::LateOuterSum in ginn/node/prod.h).
+long scenario_late_sum_columns() { return static_cast<long>(internal::late_outer_sum_columns().load()); }
+
 int scenario_mlp(int dtype, int batch, int n_layers, const int* dims, const int* acts, const float* x,
                  const int* labels, const float* const* W, const float* const* b, int iters, float* out_loss,
                  float* out_nll, float* const* dW, float* const* db, float* out_ms) {

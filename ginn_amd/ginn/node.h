@@ -313,6 +313,9 @@ inline std::atomic<size_t>& lazy_grad_settles() {
 // launches, partial sums and their fold; nothing reads such a gradient before
 // the pass ends, so while a window is open the nodes postpone those folds
 // (ginn_hip_defer_folds) and the pass runs them all as one launch at its end.
+// Other work that only the end of the pass needs registers itself with
+// at_close() (the gradient of a left operand shared by many merged products,
+// node/prod.h).
 class FoldWindow {
   static int& depth() {
     thread_local int d = 0;
@@ -322,13 +325,23 @@ class FoldWindow {
     thread_local std::vector<ginn_hip_ctx*> v;
     return v;
   }
+  // fn(run): run != 0 does the postponed work, run == 0 only forgets it.
+  static std::vector<void (*)(int)>& hooks() {
+    thread_local std::vector<void (*)(int)> v;
+    return v;
+  }
 
  public:
   FoldWindow() { ++depth(); }
   FoldWindow(const FoldWindow&) = delete;
   FoldWindow& operator=(const FoldWindow&) = delete;
   ~FoldWindow() {
-    if (--depth() == 0 && !touched().empty()) {  // left by an exception: nothing stays queued
+    if (--depth() != 0) return;
+    if (!hooks().empty()) {  // left by an exception: nothing stays queued
+      for (auto* fn : hooks()) fn(0);
+      hooks().clear();
+    }
+    if (!touched().empty()) {
       for (ginn_hip_ctx* c : touched()) (void)ginn_hip_flush_folds(c);
       touched().clear();
     }
@@ -338,9 +351,23 @@ class FoldWindow {
     auto& v = touched();
     if (std::find(v.begin(), v.end(), ctx) == v.end()) v.push_back(ctx);
   }
+  static void at_close(void (*fn)(int)) {
+    auto& v = hooks();
+    if (std::find(v.begin(), v.end(), fn) == v.end()) v.push_back(fn);
+  }
   // The end of the pass: the outermost window folds what was postponed.
   void close() {
     if (depth() != 1) return;
+    std::vector<void (*)(int)> fns;
+    fns.swap(hooks());
+    for (size_t i = 0; i < fns.size(); ++i) {
+      try {
+        fns[i](1);
+      } catch (...) {
+        for (size_t j = i + 1; j < fns.size(); ++j) fns[j](0);
+        throw;
+      }
+    }
     std::vector<ginn_hip_ctx*> v;
     v.swap(touched());
     for (ginn_hip_ctx* c : v) GINN_HIP_CALL(ginn_hip_flush_folds(c));

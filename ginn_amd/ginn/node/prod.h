@@ -3,6 +3,7 @@
 #define GINN_NODE_PROD_H
 
 #include <algorithm>
+#include <atomic>
 
 #include <ginn/node/data.h>
 #include <ginn/nonlin.h>
@@ -105,6 +106,50 @@ class ColumnTable {
   }
 };
 
+// The gradient of a left operand that many merged products share (the weight
+// matrix of a recurrent cell: one merged product per time step, each adding
+// dY_t X_t^T, ginn/node/prod.h:57-63).  Nothing reads a leaf's gradient before
+// the backward pass ends, so while a pass is running (FoldWindow) the products
+// only list their columns here and the end of the pass runs ONE product that
+// sums over the columns of all of them (ginn_hip_gemm_outer_sum).  The tables
+// belong to the node that queued first; in a graph that is run again with its
+// tensors in place they are the same every pass and nothing is uploaded.
+struct LateOuterSum {
+  void* target;
+  ginn_hip_ctx* ctx;
+  DevPtr dev;
+  ginn_hip_dtype dtype;
+  Size m, n;
+  float beta;
+  ColumnTable* a_cols;
+  ColumnTable* b_cols;
+};
+inline std::vector<LateOuterSum>& late_outer_sums() {
+  thread_local std::vector<LateOuterSum> jobs;
+  return jobs;
+}
+// Columns summed by postponed products so far (process-wide, for tests).
+inline std::atomic<size_t>& late_outer_sum_columns() {
+  static std::atomic<size_t> n{0};
+  return n;
+}
+inline void run_late_outer_sums(int run) {
+  std::vector<LateOuterSum> jobs;
+  jobs.swap(late_outer_sums());
+  if (!run) return;
+  for (LateOuterSum& j : jobs) {
+    const size_t k = j.a_cols->size();
+    GINN_ASSERT(k == j.b_cols->size());
+    const int aligned = j.a_cols->aligned() && j.b_cols->aligned();
+    auto* ta = static_cast<const void* const*>(j.a_cols->commit(j.dev, j.ctx));
+    auto* tb = static_cast<const void* const*>(j.b_cols->commit(j.dev, j.ctx));
+    GINN_HIP_CALL(ginn_hip_gemm_outer_sum(j.ctx, j.dtype, static_cast<int>(j.m), static_cast<int>(j.n),
+                                          static_cast<int>(k), ta, tb, j.beta, j.target, static_cast<int>(j.m),
+                                          aligned));
+    late_outer_sum_columns() += k;
+  }
+}
+
 }  // namespace internal
 
 // Y = A * [B_0 B_1 ... ]: the product Autobatch forms from products that share
@@ -121,6 +166,34 @@ class GatherProdNode : public BaseDataNode<Scalar>, public ColumnPartition {
   std::vector<NodePtr<Scalar>> bs_;
   std::vector<Size> offsets_, extents_;
   internal::ColumnTable values_, grads_;
+  internal::ColumnTable sum_a_, sum_b_;  // of the left operand's postponed gradient, when this node queued first
+
+  // Lists dY's and the right operands' columns for the product that forms the
+  // left operand's gradient at the end of the pass; false: form it now.
+  bool postpone_left_gradient(ginn_hip_ctx* ctx, Size m, Size k, Size total) {
+    using namespace internal;
+    if (!FoldWindow::open() || !a_->inputs().empty()) return false;
+    auto& jobs = late_outer_sums();
+    void* target = nullptr;
+    LateOuterSum* job = nullptr;
+    for (auto& j : jobs)
+      if (j.target == a_->grad_storage().data()) job = &j;
+    if (job) {
+      if (job->ctx != ctx || job->dtype != dtype_of<Scalar>() || job->m != m || job->n != k || job->dev != dev())
+        return false;
+    } else {
+      const bool fresh = a_->take_lazy_zero();
+      target = a_->grad().data();
+      sum_a_.begin();
+      sum_b_.begin();
+      jobs.push_back({target, ctx, dev(), dtype_of<Scalar>(), m, k, fresh ? 0.f : 1.f, &sum_a_, &sum_b_});
+      job = &jobs.back();
+      FoldWindow::at_close(&run_late_outer_sums);
+    }
+    job->a_cols->add(grad().data(), total, static_cast<size_t>(m) * sizeof(Scalar));
+    for (auto& b : bs_) job->b_cols->add(b->value().data(), b->value().cols(), static_cast<size_t>(k) * sizeof(Scalar));
+    return true;
+  }
 
   void forward_() override {
     internal::require_gpu(dev(), "GatherProd");
@@ -153,7 +226,7 @@ class GatherProdNode : public BaseDataNode<Scalar>, public ColumnPartition {
     const Size m = a.rows(), k = a.cols(), total = value().cols();
     if (m == 0 || total == 0 || k == 0) return;
     ginn_hip_ctx* ctx = internal::ctx_of(value());
-    if (a_->has_grad()) {
+    if (a_->has_grad() && !postpone_left_gradient(ctx, m, k, total)) {
       // dA[m x k] += dY[m x total] * X^T, X's columns gathered: they are the
       // stored columns of the transposed operand, indexed along the sum.
       auto* table = static_cast<const void* const*>(values_.commit(dev(), ctx));

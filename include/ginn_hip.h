@@ -242,6 +242,21 @@ int ginn_hip_gemm_gathered(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
                            void* C, int ldc, void* const* dev_c_cols,
                            int cols_aligned);
 
+/* C[m x n] = sum_{j < k} a_j b_j^T + beta * C: a sum of outer products of
+ * scattered columns, a_j (m elements) at dev_a_cols[j], b_j (n elements) at
+ * dev_b_cols[j]; both tables are DEVICE arrays of k entries.  A shared left
+ * operand W of several products Y_t = W X_t receives dW += dY_t X_t^T from
+ * each of them (ProdNode::backward_, ginn/node/prod.h:57-63; for the products
+ * Autobatch merges, ginn/autobatch.h:149-183, once per merged group): with
+ * the columns of all dY_t and all X_t listed in the two tables this is ONE
+ * product that sums over every column of every use, run once at the end of
+ * the backward pass.  cols_aligned != 0 promises 16-byte aligned column
+ * bases.  C is dense (ldc >= m). */
+int ginn_hip_gemm_outer_sum(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int m,
+                            int n, int k, const void* const* dev_a_cols,
+                            const void* const* dev_b_cols, float beta,
+                            void* C, int ldc, int cols_aligned);
+
 /* out[c] = sum_r x[r, c] * y[r, c] + beta * out[c] for `cols` columns of
  * height `rows` (contiguous, ld = rows).  This is the degenerate m = n = 1
  * batched product that SoftmaxOp::backward (ginn/nonlin.h:177-184) and

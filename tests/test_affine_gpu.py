@@ -353,6 +353,48 @@ def test_gathered_gemm(dev, dt, m, k, n, misalign):
     assert np.isnan(flat[mask]).all()
 
 
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(96, 72, 40), (64, 64, 300), (130, 33, 7), (1024, 384, 1500), (8, 12, 1), (5, 3, 0)])
+@pytest.mark.parametrize("misalign", [False, True])
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_outer_sum_of_scattered_columns(dev, dt, m, n, k, misalign, beta):
+    """ginn_hip_gemm_outer_sum: dW = sum_j dy_j x_j^T + beta dW over column
+    pairs that lie anywhere -- what the accumulating dA += dY B^T of every
+    product sharing A (ginn/node/prod.h:57-63) adds up to."""
+    from gpu_util import TOL, round_to
+    rng = np.random.default_rng(m * 11 + n * 5 + k + misalign)
+    dY = round_to(rng.standard_normal((m, max(k, 1))) / np.sqrt(max(k, 1)), dt)[:, :k]
+    X = round_to(rng.standard_normal((n, max(k, 1))), dt)[:, :k]
+    dW0 = round_to(rng.standard_normal((m, n)), dt)
+    vp = ctypes.c_void_p
+    table_a = table_b = None
+    if k > 0:
+        keep_a, _, _, table_a = _scatter_columns(dev, dY, dt, rng, misalign)
+        keep_b, _, _, table_b = _scatter_columns(dev, X, dt, rng, misalign)
+    start = dW0 if beta else np.full((m, n), np.nan, np.float32)
+    bw, pw, ldw = dev.put(start, dt)
+    dev.lib.call("ginn_hip_gemm_outer_sum", dev.ctx, dt, m, n, k, vp(table_a) if k else None,
+                 vp(table_b) if k else None, beta, vp(pw), ldw, 0 if misalign else 1)
+    dev.sync()
+    want = dY.astype(np.float64) @ X.astype(np.float64).T + (dW0 if beta else 0)
+    got = dev.get(bw, (m, n), ldw)
+    if k == 0 and not beta:
+        assert (got == 0).all()
+    else:
+        assert rel_fro(got, want) <= TOL[dt]
+
+
+def test_outer_sum_argument_checks(dev):
+    vp = ctypes.c_void_p
+    b, p, ld = dev.put(np.zeros((8, 8), np.float32), capi.F32)
+    with pytest.raises(capi.GinnHipError, match="NULL table"):
+        dev.lib.call("ginn_hip_gemm_outer_sum", dev.ctx, capi.F32, 8, 8, 4, None, vp(p), 0.0, vp(p), 8, 1)
+    with pytest.raises(capi.GinnHipError, match="ldc"):
+        dev.lib.call("ginn_hip_gemm_outer_sum", dev.ctx, capi.F32, 8, 8, 4, vp(p), vp(p), 0.0, vp(p), 4, 1)
+    with pytest.raises(capi.GinnHipError, match="C is NULL"):
+        dev.lib.call("ginn_hip_gemm_outer_sum", dev.ctx, capi.F32, 8, 8, 4, vp(p), vp(p), 0.0, None, 8, 1)
+
+
 def test_gathered_gemm_argument_checks(dev):
     vp = ctypes.c_void_p
     b, p, ld = dev.put(np.zeros((8, 8), np.float32), capi.F32)

@@ -26,6 +26,7 @@ def shim():
     lib = ctypes.CDLL(str(SHIM))
     lib.scenario_last_error.restype = ctypes.c_char_p
     lib.scenario_timed_fills.restype = ctypes.c_long
+    lib.scenario_late_sum_columns.restype = ctypes.c_long
     return lib
 
 
@@ -301,9 +302,13 @@ def test_lstm_level_executor_full_config(shim, gather):
     """256 sequences, lengths U{5..40}: ~100 k nodes in a few thousand launches."""
     rng = np.random.default_rng(2024)
     lens = rng.integers(5, 41, 256).tolist()
+    late = shim.scenario_late_sum_columns()
     got, want, stats = run_lstm(shim, 3, lens, 128, 256, seed=9)
     compare_lstm(got, want)
     assert stats["launches"] < stats["nodes"] / 10
+    # With gathered products the weight gradient is ONE product per pass over the columns of all
+    # steps (the warm-up pass and the timed one); with the reference's concatenation it is one per step.
+    assert shim.scenario_late_sum_columns() - late == (2 * sum(lens) if gather else 0)
     got, want, stats = run_lstm(shim, 7, lens, 128, 256, seed=9, iters=3)
     compare_lstm(got, want)
     assert shim.scenario_timed_fills() == 0  # no gradient was zeroed on demand, one launch each
