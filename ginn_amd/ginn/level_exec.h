@@ -50,6 +50,7 @@ class LevelExecutor {
     size_t zero_max = 0;         // set: zero fill of `count` regions (pointers at offset, byte counts at aux)
     size_t aux = 0;
     size_t mixed_max = 0;        // set: `count` operation records at offset, the longest of this many elements
+    bool late = false;           // a reduction that runs as part of one at the end of the pass (LateReduce)
   };
   // What one flush (the described nodes of one level and pass) turned into.
   // As long as the nodes describe the same operations on the same memory --
@@ -80,6 +81,21 @@ class LevelExecutor {
     long plan;
     size_t index;
   };
+  // The reductions of a frozen backward pass into the gradient of one leaf (a
+  // bias that every step of every sequence adds to: one reduction per level)
+  // as ONE reduction over all their sources at the end of the pass.  Nothing
+  // reads a leaf's gradient during the pass, and a source that is gradient
+  // storage owned by its node is not written again once that node has run
+  // (only nodes above it can alias it), so the sum is the same.
+  struct LateReduce {
+    void* dst = nullptr;
+    int dtype = GINN_HIP_F32;
+    size_t n = 0;
+    std::vector<const void*> srcs;
+    std::vector<Launch*> members;
+    void* dev = nullptr;
+  };
+  std::vector<LateReduce> late_reduces_;
   std::vector<Chain> chains_;
   std::vector<Item> fused_[3];
   bool fused_ready_ = false;
@@ -253,6 +269,7 @@ class LevelExecutor {
   void launch(const Plan& plan) { launch(plan, 0, plan.launches.size()); }
 
   void launch(const Plan& plan, size_t first, size_t count) {
+    size_t skipped = 0;
     for (size_t li = first; li < first + count; ++li) {
       const Launch& l = plan.launches[li];
       if (l.zero_max) {
@@ -262,6 +279,10 @@ class LevelExecutor {
         continue;
       }
       if (l.reduce_dst) {
+        if (l.late) {
+          ++skipped;
+          continue;
+        }
         GINN_HIP_CALL(ginn_hip_multi_reduce(ctx_, static_cast<ginn_hip_dtype>(l.key.dtype), l.key.n,
                                             static_cast<int>(l.count),
                                             static_cast<const void* const*>(plan.dev) + l.offset, l.reduce_dst, 1));
@@ -272,7 +293,102 @@ class LevelExecutor {
           reinterpret_cast<const ginn_hip_multi_op*>(static_cast<const void* const*>(plan.dev) + l.offset),
           l.mixed_max));
     }
-    launches_ += count;
+    launches_ += count - skipped;
+  }
+
+  // Gradient storage [begin, end) of a node, whatever its scalar.
+  static bool grad_range(BaseNode& n, uintptr_t& begin, uintptr_t& end) {
+    auto of = [&](auto* t) {
+      if (!t) return false;
+      auto& g = t->grad_storage();
+      begin = reinterpret_cast<uintptr_t>(g.data());
+      end = begin + static_cast<size_t>(g.size()) * sizeof(*g.data());
+      return true;
+    };
+    return of(dynamic_cast<Node<Real>*>(&n)) || of(dynamic_cast<Node<Half>*>(&n)) ||
+           of(dynamic_cast<Node<BFloat16>*>(&n));
+  }
+
+  void drop_late_reductions() {
+    for (LateReduce& r : late_reduces_) {
+      for (Launch* l : r.members) l->late = false;
+      if (r.dev) {
+        try {
+          dev_->free(r.dev);
+        } catch (...) {
+        }
+      }
+    }
+    late_reduces_.clear();
+  }
+
+  // freeze(): see LateReduce.
+  void plan_late_reductions() {
+    drop_late_reductions();
+    std::vector<std::pair<uintptr_t, uintptr_t>> owned;  // gradient storage that belongs to its node
+    std::vector<uintptr_t> leaves;                        // ... of nodes without inputs
+    for (auto& n : list_) {
+      if (!n->has_grad() || !n->owns_grad()) continue;
+      uintptr_t b = 0, e = 0;
+      if (!grad_range(*n, b, e) || b == e) continue;
+      owned.emplace_back(b, e);
+      if (n->ins().empty()) leaves.push_back(b);
+    }
+    std::sort(owned.begin(), owned.end());
+    std::sort(leaves.begin(), leaves.end());
+    auto is_owned = [&](const void* p, size_t bytes) {
+      const uintptr_t at = reinterpret_cast<uintptr_t>(p);
+      auto it = std::upper_bound(owned.begin(), owned.end(), std::make_pair(at, ~uintptr_t(0)));
+      if (it == owned.begin()) return false;
+      --it;
+      return at >= it->first && at + bytes <= it->second;
+    };
+    for (const Step& step : steps_[kBackward]) {
+      if (step.plan < 0) continue;
+      Plan& plan = plans_[kBackward][static_cast<size_t>(step.plan)];
+      for (Launch& l : plan.launches) {
+        if (!l.reduce_dst) continue;
+        if (!std::binary_search(leaves.begin(), leaves.end(), reinterpret_cast<uintptr_t>(l.reduce_dst))) continue;
+        const size_t bytes = l.key.n * (l.key.dtype == GINN_HIP_F32 ? 4 : 2);
+        bool ok = true;
+        for (size_t i = 0; i < l.count && ok; ++i) ok = is_owned(plan.blob[l.offset + i], bytes);
+        if (!ok) continue;
+        LateReduce* into = nullptr;
+        for (LateReduce& r : late_reduces_)
+          if (r.dst == l.reduce_dst && r.dtype == l.key.dtype && r.n == l.key.n) into = &r;
+        if (!into) {
+          late_reduces_.emplace_back();
+          into = &late_reduces_.back();
+          into->dst = l.reduce_dst;
+          into->dtype = l.key.dtype;
+          into->n = l.key.n;
+        }
+        into->srcs.insert(into->srcs.end(), plan.blob.begin() + static_cast<long>(l.offset),
+                          plan.blob.begin() + static_cast<long>(l.offset + l.count));
+        into->members.push_back(&l);
+      }
+    }
+    // One reduction alone gains nothing by waiting.
+    late_reduces_.erase(std::remove_if(late_reduces_.begin(), late_reduces_.end(),
+                                       [](const LateReduce& r) {
+                                         return r.members.size() < 2 || r.srcs.size() > 0x7fffffffu;
+                                       }),
+                        late_reduces_.end());
+    for (LateReduce& r : late_reduces_) {
+      r.dev = dev_->alloc(r.srcs.size() * sizeof(void*));
+      GINN_HIP_CALL(ginn_hip_memcpy_h2d(ctx_, r.dev, r.srcs.data(), r.srcs.size() * sizeof(void*)));
+      for (Launch* l : r.members) l->late = true;
+    }
+    if (!late_reduces_.empty()) GINN_HIP_CALL(ginn_hip_sync(ctx_));  // pageable copies: the tables have arrived
+  }
+
+  void run_late_reductions() {
+    for (const LateReduce& r : late_reduces_) {
+      GINN_HIP_CALL(ginn_hip_multi_reduce(ctx_, static_cast<ginn_hip_dtype>(r.dtype), r.n,
+                                          static_cast<int>(r.srcs.size()),
+                                          static_cast<const void* const*>(r.dev), r.dst, 1));
+      ++launches_;
+    }
   }
 
   // Ends a step: launches what its nodes described (reusing the plan of the
@@ -546,7 +662,7 @@ class LevelExecutor {
           end_run();
           emit_launch(ref);
         } else if (l.reduce_dst) {
-          reductions.emplace_back(ref, static_cast<int>(run.size()));
+          if (!l.late) reductions.emplace_back(ref, static_cast<int>(run.size()));
         } else {
           run.push_back(ref);
         }
@@ -603,6 +719,7 @@ class LevelExecutor {
   ~LevelExecutor() {
     drop_graph();
     drop_chains();
+    drop_late_reductions();
     for (auto& pass : plans_)
       for (auto& plan : pass)
         if (plan.dev) {
@@ -624,6 +741,7 @@ class LevelExecutor {
     GINN_ASSERT(!unplanned_fill_,
                 "LevelExecutor::freeze(): a node that declares GradUse::Overwrites added to a gradient that "
                 "reset_grad() had only flagged; run with set_lazy_grad_reset(false)");
+    plan_late_reductions();
     frozen_ = true;
     return *this;
   }
@@ -631,6 +749,7 @@ class LevelExecutor {
     frozen_ = false;
     drop_graph();
     drop_chains();
+    drop_late_reductions();
     return *this;
   }
   // fuse(): on a frozen executor, joins the table launches of consecutive
@@ -771,6 +890,7 @@ class LevelExecutor {
         }
       }
       for (BaseNode* n : lazy_direct_) n->clear_lazy_zero();  // all taken already, unless a node returned early
+      run_late_reductions();
       folds.close();
       return *this;
     }
