@@ -381,6 +381,10 @@ int launch_gemm_generic(ginn_hip_ctx* ctx, const GemmArgs& args);
 // (without setting an error) when the shape does not qualify.
 int launch_gemm_fast16(ginn_hip_ctx* ctx, const GemmArgs& args);
 
+// fp32 products with at most a few hundred 32 x 32 output tiles: K split over
+// the 16 waves of a workgroup, one launch; kUnsupported otherwise.
+int launch_gemm_ksplit(ginn_hip_ctx* ctx, const GemmArgs& args);
+
 // Bandwidth-oriented kernel for narrow right-hand sides (n <= 64).
 int launch_gemm_skinny(ginn_hip_ctx* ctx, const GemmArgs& args);
 int launch_gemm_skinny_mfma(ginn_hip_ctx* ctx, const GemmArgs& args);

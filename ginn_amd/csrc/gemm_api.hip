@@ -59,6 +59,8 @@ int launch_gemm(ginn_hip_ctx* ctx, const GemmArgs& a) {
   int rc = kUnsupported;
   if (a.dtype != GINN_HIP_F32 && a.batch == 1 && a.n <= 8) rc = launch_gemm_mid(ctx, a);
   if (rc != kUnsupported) return rc;
+  rc = launch_gemm_ksplit(ctx, a);
+  if (rc != kUnsupported) return rc;
   rc = launch_gemm_skinny(ctx, a);
   if (rc != kUnsupported) return rc;
   rc = launch_gemm_fast16(ctx, a);
@@ -222,6 +224,7 @@ int ginn_hip_gemm_gathered(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
   GH_HIP(hipSetDevice(ctx->device));
   // Without a table this is an ordinary product and takes the ordinary route.
   if (!a.bcols && !a.ccols) return launch_gemm(ctx, a);
+  if (int rc = launch_gemm_ksplit(ctx, a); rc != kUnsupported) return rc;
   return launch_gemm_generic(ctx, a);
 }
 
@@ -253,6 +256,7 @@ int ginn_hip_gemm_outer_sum(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int m, int 
   if (m == 0 || n == 0) return kOk;
   GH_HIP(hipSetDevice(ctx->device));
   if (k == 0) return launch_gemm(ctx, a);
+  if (int rc = launch_gemm_ksplit(ctx, a); rc != kUnsupported) return rc;
   return launch_gemm_generic(ctx, a);
 }
 

@@ -1,0 +1,281 @@
+// fp32 products with a small output: one launch, the sum over K split inside
+// the workgroup.  The merged products of an autobatched recurrent cell
+// (ginn/autobatch.h:149-183: W [1024 x 384] times the states of the sequences
+// still alive, and its gradients) have a few hundred 32 x 32 output tiles at
+// most.  Tiles of 64 x 64 with K split over workgroups fill the machine but
+// need a second launch that folds the partial sums, which costs as much as
+// the product itself (4 us against 7).  Here a workgroup of 16 waves owns one
+// 32 x 32 tile, every wave walks one sixteenth of K with operands straight
+// from memory in the matrix instruction's own layout (no staging, no barrier
+// in the loop), and the 16 partial tiles meet in LDS, always in the same order.
+#include "common.h"
+
+namespace ginn_hip {
+namespace {
+namespace ksplit {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+// Loads through pointers of the global address space: the compiler then issues
+// global loads, which do not count against the LDS counter as flat loads do.
+typedef const float __attribute__((address_space(1)))* gfloat;
+typedef const f32x4 __attribute__((address_space(1)))* gfloat4;
+typedef const float* const __attribute__((address_space(1)))* gtable;
+__device__ __forceinline__ float gload(const float* p) { return *(gfloat)p; }
+__device__ __forceinline__ f32x4 gload4(const float* p) { return *(gfloat4)p; }
+__device__ __forceinline__ const float* gload_ptr(const float* const* p) { return *(gtable)p; }
+
+constexpr int kWaves = 16;
+constexpr int kThreads = kWaves * 64;
+constexpr int kTile = 32;
+constexpr int kStep = 16;   // values of K per step of a wave: 8 matrix instructions
+constexpr int kDepth = 4;   // steps whose operands are on their way
+// A K-contiguous operand is read as 64-byte runs (4 lanes per row, 16 rows per
+// load) and turned into the matrix instruction's layout (one row per lane)
+// through a slice of LDS that belongs to the wave: [32 rows][4 vectors of 4],
+// vector q of row r at position q ^ ((r >> 2) & 3) (no bank conflicts either way).
+constexpr int kStageFloats = kTile * kStep;
+static_assert(2 * kStageFloats == kTile * kTile, "the staging slices and the partial tiles share the LDS");
+
+struct Params {
+  const float* A;
+  const float* B;
+  float* C;
+  int m, n, k;
+  int lda, ldb, ldc;
+  float beta;
+  const float* bias;
+  float* pre;
+  int act;
+  const float* const* acols;  // A by stored columns (op_a N only)
+  const float* const* bcols;  // B by stored columns
+  float* const* ccols;        // C by columns
+  int k_per_wave;             // a multiple of kStep
+};
+
+// One operand of a wave: 32 rows of op(X) (rows of A, columns of B).  KC: K is
+// the contiguous dimension in memory.  TABLE: the stored columns are given by
+// their addresses.  Every load is unconditional from a clamped, valid address;
+// what lies outside the operand is zeroed when the values are used, so that
+// nothing waits for a load where it is issued.
+template <bool KC, bool TABLE>
+struct Operand {
+  const float* row_lo = nullptr;  // KC: rows lane / 4 and lane / 4 + 16 (clamped)
+  const float* row_hi = nullptr;
+  const float* base = nullptr;    // otherwise: the lane's row (clamped) in the first stored column
+  const float* const* cols = nullptr;
+  long long ld = 0;
+  int row = 0;
+  bool ok = false;  // row lane % 32 lies inside the operand
+
+  __device__ __forceinline__ void init(const float* X, int ld_, const float* const* table, int first, int extent,
+                                       int lane) {
+    ld = ld_;
+    cols = table;
+    ok = first + (lane & 31) < extent;
+    if (KC) {
+      const int lo = min(first + (lane >> 2), extent - 1), hi = min(first + (lane >> 2) + 16, extent - 1);
+      row_lo = TABLE ? gload_ptr(table + lo) : X + lo * ld;
+      row_hi = TABLE ? gload_ptr(table + hi) : X + hi * ld;
+    } else {
+      row = min(first + (lane & 31), extent - 1);
+      base = TABLE ? nullptr : X + row;
+    }
+  }
+
+  // The lane's share of K = j .. j + 15, j < k_end.  KC: values
+  // j + 4 (lane % 4) + 0 .. 3 of its two rows; otherwise the eight values
+  // j + 8 (lane / 32) + t of its row.  Positions beyond k_end repeat earlier ones.
+  __device__ __forceinline__ void fetch(int j, int k_end, int lane, float (&v)[8]) const {
+    if (KC) {
+      // k_end is a multiple of 4 (the launcher sees to it): a vector that would
+      // begin beyond it repeats the last one.
+      const int kk = min(j + 4 * (lane & 3), k_end - 4);
+      const f32x4 lo = gload4(row_lo + kk);
+      const f32x4 hi = gload4(row_hi + kk);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        v[t] = lo[t];
+        v[4 + t] = hi[t];
+      }
+    } else {
+      const int kk = j + 8 * (lane >> 5);
+      const float* from[8];
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const int at = min(kk + t, k_end - 1);
+        from[t] = TABLE ? gload_ptr(cols + at) + row : base + at * ld;
+      }
+#pragma unroll
+      for (int t = 0; t < 8; ++t) v[t] = gload(from[t]);
+    }
+  }
+
+  // v as the matrix instruction wants it: the eight values K = j + 8 (lane / 32) + t
+  // of row lane % 32, zero outside the operand.  KC: through the wave's own LDS
+  // slice (a wave's LDS accesses execute in order, so no barrier is needed
+  // between this step's reads and the next step's writes).
+  __device__ __forceinline__ void arrange(float* stage, int j, int k_end, int lane, float (&v)[8]) const {
+    if (KC) {
+      const int srow = lane >> 2, q = lane & 3;
+      const int swz = (srow >> 2) & 3;  // the same for srow and srow + 16
+      *reinterpret_cast<f32x4*>(stage + srow * kStep + ((q ^ swz) << 2)) = f32x4{v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<f32x4*>(stage + (srow + 16) * kStep + ((q ^ swz) << 2)) = f32x4{v[4], v[5], v[6], v[7]};
+      const int r = lane & 31, h = lane >> 5, rs = (r >> 2) & 3;
+      const f32x4 q0 = *reinterpret_cast<const f32x4*>(stage + r * kStep + (((2 * h) ^ rs) << 2));
+      const f32x4 q1 = *reinterpret_cast<const f32x4*>(stage + r * kStep + (((2 * h + 1) ^ rs) << 2));
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        v[t] = q0[t];
+        v[4 + t] = q1[t];
+      }
+    }
+    const int kk = j + 8 * (lane >> 5);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) v[t] = ok && kk + t < k_end ? v[t] : 0.f;
+  }
+};
+
+template <bool AKC, bool BKC, bool ATAB, bool BTAB>
+__global__ __launch_bounds__(kThreads) void gemm_ksplit_kernel(Params p) {
+  __shared__ __align__(16) float lds[kWaves * kTile * kTile];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register: K ranges and branches are per wave
+  const int m0 = blockIdx.x * kTile, n0 = blockIdx.y * kTile;
+  Operand<AKC, ATAB> opa;
+  Operand<BKC, BTAB> opb;
+  opa.init(p.A, p.lda, p.acols, m0, p.m, lane);
+  opb.init(p.B, p.ldb, p.bcols, n0, p.n, lane);
+  float* stage_a = lds + wave * 2 * kStageFloats;
+  float* stage_b = stage_a + kStageFloats;
+  const int k_begin = wave * p.k_per_wave;
+  const int k_end = min(p.k, k_begin + p.k_per_wave);
+
+  f32x16 acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+  if (k_begin < k_end) {
+    // A matrix instruction multiplies 32 x 2 by 2 x 32: lanes 0-31 supply one
+    // value of K, lanes 32-63 another.  Half h of the wave takes K = j + 8 h + t
+    // in the t-th of a step's eight instructions.
+    float a[kDepth][8], b[kDepth][8];
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+      if (k_begin + kStep * d < k_end) {
+        opa.fetch(k_begin + kStep * d, k_end, lane, a[d]);
+        opb.fetch(k_begin + kStep * d, k_end, lane, b[d]);
+      }
+    }
+    for (int j = k_begin; j < k_end; j += kStep * kDepth) {
+#pragma unroll
+      for (int d = 0; d < kDepth; ++d) {
+        if (j + kStep * d < k_end) {
+          opa.arrange(stage_a, j + kStep * d, k_end, lane, a[d]);
+          opb.arrange(stage_b, j + kStep * d, k_end, lane, b[d]);
+#pragma unroll
+          for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[d][t], b[d][t], acc, 0, 0, 0);
+          const int next = j + kStep * (d + kDepth);
+          if (next < k_end) {
+            opa.fetch(next, k_end, lane, a[d]);
+            opb.fetch(next, k_end, lane, b[d]);
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();  // the partial tiles take the place of the staging slices
+  // Accumulator element 4 q + i of a lane is row 8 q + 4 h + i of column r.
+  // A column's 32 rows lie in 8 chunks of 4; chunk c of column r sits at
+  // position c ^ (r & 7), which spreads the 16-byte stores of a wave over all banks.
+  {
+    const int r = lane & 31, h = lane >> 5;
+    float* mine = lds + wave * kTile * kTile;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int chunk = 2 * q + h;
+      f32x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = acc[4 * q + i];
+      *reinterpret_cast<f32x4*>(mine + r * kTile + ((chunk ^ (r & 7)) << 2)) = v;
+    }
+  }
+  __syncthreads();
+  const int row = threadIdx.x & 31, col = threadIdx.x >> 5;
+  const int at = col * kTile + ((((row >> 2) ^ (col & 7)) << 2) | (row & 3));
+  float sum = 0.f;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) sum += lds[w * kTile * kTile + at];
+  const int grow = m0 + row, gcol = n0 + col;
+  if (grow >= p.m || gcol >= p.n) return;
+  const long long off = static_cast<long long>(gcol) * p.ldc + grow;
+  float* out = p.ccols ? p.ccols[gcol] + grow : p.C + off;
+  float* keep = p.pre ? p.pre + off : nullptr;
+  if (p.beta != 0.f) sum += p.beta * (keep ? *keep : *out);
+  if (p.bias) sum += p.bias[grow];
+  if (keep) *keep = sum;
+  if (p.act != GINN_HIP_ACT_IDENTITY) sum = act_forward<kFastMath<F32>>(p.act, sum);
+  *out = sum;
+}
+
+template <bool AKC, bool BKC>
+int launch_layout(ginn_hip_ctx* ctx, const Params& p, dim3 grid) {
+  // Column tables: A only when its columns are what is stored (op_a N).
+  if (!AKC && p.acols) {
+    if (p.bcols) gemm_ksplit_kernel<AKC, BKC, true, true><<<grid, kThreads, 0, ctx->stream>>>(p);
+    else gemm_ksplit_kernel<AKC, BKC, true, false><<<grid, kThreads, 0, ctx->stream>>>(p);
+  } else {
+    if (p.bcols) gemm_ksplit_kernel<AKC, BKC, false, true><<<grid, kThreads, 0, ctx->stream>>>(p);
+    else gemm_ksplit_kernel<AKC, BKC, false, false><<<grid, kThreads, 0, ctx->stream>>>(p);
+  }
+  GH_HIP(hipGetLastError());
+  return kOk;
+}
+
+}  // namespace ksplit
+}  // namespace
+
+int launch_gemm_ksplit(ginn_hip_ctx* ctx, const GemmArgs& a) {
+  using namespace ksplit;
+  if (a.dtype != GINN_HIP_F32 || a.batch != 1) return kUnsupported;
+  if (a.pre && a.ccols) return kUnsupported;
+  // Every wave reads its share of both operand panels itself: that pays while a
+  // wave's share of K is what it asks for at once (kDepth steps) and there is
+  // one workgroup per CU at most.  Longer sums and larger outputs belong to the
+  // kernels that share operands through LDS.
+  if (a.k < 32 || a.k > kWaves * kStep * kDepth) return kUnsupported;
+  const long long tiles = static_cast<long long>((a.m + kTile - 1) / kTile) * ((a.n + kTile - 1) / kTile);
+  if (tiles > ctx->num_cus) return kUnsupported;
+  // A narrow right-hand side under a left operand of several MiB is one pass over that operand at
+  // memory speed: the skinny kernels' case.
+  if (a.n <= 16 && static_cast<long long>(a.m) * a.k > (1ll << 20)) return kUnsupported;
+  const bool akc = a.op_a == GINN_HIP_OP_T, bkc = a.op_b == GINN_HIP_OP_N;
+  if (a.acols && akc) return kUnsupported;
+  Params p;
+  p.A = static_cast<const float*>(a.A);
+  p.B = static_cast<const float*>(a.B);
+  p.C = static_cast<float*>(a.C);
+  p.m = a.m;
+  p.n = a.n;
+  p.k = a.k;
+  p.lda = a.lda;
+  p.ldb = a.ldb;
+  p.ldc = a.ldc;
+  p.beta = a.beta;
+  p.bias = static_cast<const float*>(a.bias);
+  p.pre = static_cast<float*>(a.pre);
+  p.act = a.act;
+  p.acols = reinterpret_cast<const float* const*>(a.acols);
+  p.bcols = reinterpret_cast<const float* const*>(a.bcols);
+  p.ccols = reinterpret_cast<float* const*>(a.ccols);
+  p.k_per_wave = ((a.k + kWaves - 1) / kWaves + kStep - 1) / kStep * kStep;
+  // K-contiguous operands are read as 16-byte vectors, also at the end of K.
+  if ((akc || bkc) && a.k % 4 != 0) return kUnsupported;
+  auto aligned = [](const void* ptr, int ld) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && ld % 4 == 0; };
+  if (akc && !aligned(a.A, a.lda)) return kUnsupported;
+  if (bkc && !(a.bcols ? a.cols_vec_ld : aligned(a.B, a.ldb))) return kUnsupported;
+  const dim3 grid((a.m + kTile - 1) / kTile, (a.n + kTile - 1) / kTile);
+  if (akc) return bkc ? launch_layout<true, true>(ctx, p, grid) : launch_layout<true, false>(ctx, p, grid);
+  return bkc ? launch_layout<false, true>(ctx, p, grid) : launch_layout<false, false>(ctx, p, grid);
+}
+
+}  // namespace ginn_hip

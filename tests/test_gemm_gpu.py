@@ -72,7 +72,11 @@ def test_reference_prod_golden(dev, golden, dt, op_a, op_b):
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("op_a,op_b", LAYOUTS)
 @pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 5, 7), (64, 64, 64), (65, 63, 33), (128, 128, 128),
-                                   (200, 136, 72), (129, 257, 100), (10, 64, 512), (512, 64, 784)])
+                                   (200, 136, 72), (129, 257, 100), (10, 64, 512), (512, 64, 784),
+                                   # fp32: one launch with K split inside the workgroup, up to its limits
+                                   # (256 tiles of 32 x 32, K = 1024) and just beyond
+                                   (33, 31, 36), (1024, 256, 384), (384, 250, 1024), (500, 500, 1000),
+                                   (96, 40, 1028)])
 @pytest.mark.parametrize("beta", [0.0, 1.0])
 def test_small_shapes(dev, dt, op_a, op_b, m, n, k, beta):
     run_case(dev, dt, op_a, op_b, m, n, k, beta, seed=m * 7 + n * 3 + k)
