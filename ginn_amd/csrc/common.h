@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <map>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -55,10 +56,21 @@ void clear_error();
 // Free device blocks kept for reuse, by block size.  Every block is used on the
 // context's one stream only, so a block released by the host may be handed out
 // again at once: whatever still reads it was enqueued earlier on that stream.
+// Blocks of up to 64 KiB are cut from 2 MiB allocations ("slabs") of their size
+// class, next to each other in address order: a graph of a hundred thousand
+// small tensors then costs a few hundred driver allocations instead of one per
+// tensor, and tensors made one after the other share pages.
+struct ginn_hip_slab {
+  size_t block = 0;   // size class
+  size_t carved = 0;  // bytes handed out so far (blocks are cut front to back)
+  size_t live = 0;    // blocks in use; a slab without any can go back to the driver
+};
 struct ginn_hip_pool {
   std::mutex mutex;
   std::unordered_map<size_t, std::vector<void*>> free_blocks;  // block size -> blocks
   std::unordered_map<void*, size_t> block_size;                // every live or cached block of the pool
+  std::map<uintptr_t, ginn_hip_slab> slabs;                    // by base address
+  std::unordered_map<size_t, uintptr_t> open_slab;             // size class -> the slab being cut
   size_t cached_bytes = 0;
   size_t limit_bytes = size_t(8) << 30;  // beyond this, released blocks go back to the driver
   bool enabled = true;

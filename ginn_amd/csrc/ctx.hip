@@ -3,6 +3,9 @@
 #include <new>
 #include <string>
 
+#include <algorithm>
+#include <iterator>
+
 #include "common.h"
 
 namespace ginn_hip {
@@ -129,15 +132,63 @@ size_t pool_block_size(size_t bytes) {
   while (b < bytes) b <<= 1;
   return b;
 }
-// Gives every cached block back to the driver; the caller holds the pool's mutex.
+constexpr size_t kSlabBytes = size_t(2) << 20;
+constexpr size_t kSlabMaxBlock = size_t(64) << 10;
+
+// The slab that ptr was cut from, or end().
+std::map<uintptr_t, ginn_hip_slab>::iterator slab_of(ginn_hip_pool& pool, const void* ptr) {
+  const uintptr_t at = reinterpret_cast<uintptr_t>(ptr);
+  auto it = pool.slabs.upper_bound(at);
+  if (it == pool.slabs.begin()) return pool.slabs.end();
+  --it;
+  return at < it->first + kSlabBytes ? it : pool.slabs.end();
+}
+
+// Gives a slab without live blocks back to the driver (its cached blocks have
+// been taken off the free lists by the caller, or are taken off here).
+void pool_release_slab(ginn_hip_pool& pool, std::map<uintptr_t, ginn_hip_slab>::iterator slab) {
+  const uintptr_t base = slab->first;
+  const ginn_hip_slab s = slab->second;
+  auto list = pool.free_blocks.find(s.block);
+  if (list != pool.free_blocks.end()) {
+    auto& v = list->second;
+    const size_t before = v.size();
+    v.erase(std::remove_if(v.begin(), v.end(),
+                           [&](void* p) {
+                             const uintptr_t at = reinterpret_cast<uintptr_t>(p);
+                             return at >= base && at < base + kSlabBytes;
+                           }),
+            v.end());
+    pool.cached_bytes -= (before - v.size()) * s.block;
+  }
+  for (size_t off = 0; off < s.carved; off += s.block) pool.block_size.erase(reinterpret_cast<void*>(base + off));
+  auto open = pool.open_slab.find(s.block);
+  if (open != pool.open_slab.end() && open->second == base) pool.open_slab.erase(open);
+  (void)hipFree(reinterpret_cast<void*>(base));
+  pool.slabs.erase(slab);
+}
+
+// Gives every cached block that can go back to the driver: blocks of their
+// own, and slabs none of whose blocks is in use.  The caller holds the pool's mutex.
 void pool_release_cached(ginn_hip_pool& pool) {
-  for (auto& [size, blocks] : pool.free_blocks)
+  for (auto& [size, blocks] : pool.free_blocks) {
+    std::vector<void*> kept;
     for (void* p : blocks) {
+      if (slab_of(pool, p) != pool.slabs.end()) {
+        kept.push_back(p);
+        continue;
+      }
       (void)hipFree(p);
       pool.block_size.erase(p);
+      pool.cached_bytes -= size;
     }
-  pool.free_blocks.clear();
-  pool.cached_bytes = 0;
+    blocks.swap(kept);
+  }
+  for (auto it = pool.slabs.begin(); it != pool.slabs.end();) {
+    auto next = std::next(it);
+    if (it->second.live == 0) pool_release_slab(pool, it);
+    it = next;
+  }
 }
 }  // namespace
 
@@ -184,6 +235,7 @@ int ginn_hip_ctx_destroy(ginn_hip_ctx* ctx) {
   if (ctx->workspace) (void)hipFree(ctx->workspace);
   if (ctx->folds.arena) (void)hipFree(ctx->folds.arena);
   pool_release_cached(ctx->pool);
+  for (auto& slab : ctx->pool.slabs) (void)hipFree(reinterpret_cast<void*>(slab.first));  // blocks never released
   if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
   return kOk;
@@ -222,7 +274,33 @@ int ginn_hip_malloc(ginn_hip_ctx* ctx, size_t bytes, void** ptr) {
       *ptr = it->second.back();
       it->second.pop_back();
       pool.cached_bytes -= block;
+      auto slab = slab_of(pool, *ptr);
+      if (slab != pool.slabs.end()) ++slab->second.live;
       return kOk;
+    }
+    if (block <= kSlabMaxBlock) {
+      // Cut the next block of this size class's slab; a new slab when it is used up.
+      auto open = pool.open_slab.find(block);
+      auto slab = open == pool.open_slab.end() ? pool.slabs.end() : pool.slabs.find(open->second);
+      if (slab == pool.slabs.end() || slab->second.carved + block > kSlabBytes) {
+        void* base = nullptr;
+        if (hipMalloc(&base, kSlabBytes) == hipSuccess) {
+          ginn_hip_slab fresh;
+          fresh.block = block;
+          slab = pool.slabs.emplace(reinterpret_cast<uintptr_t>(base), fresh).first;
+          pool.open_slab[block] = slab->first;
+        } else {
+          (void)hipGetLastError();  // no room for a slab: a block of its own below
+          slab = pool.slabs.end();
+        }
+      }
+      if (slab != pool.slabs.end()) {
+        *ptr = reinterpret_cast<void*>(slab->first + slab->second.carved);
+        slab->second.carved += block;
+        ++slab->second.live;
+        pool.block_size[*ptr] = block;
+        return kOk;
+      }
     }
   }
   hipError_t e = hipMalloc(ptr, block);
@@ -251,7 +329,20 @@ int ginn_hip_free(ginn_hip_ctx* ctx, void* ptr) {
   auto it = pool.block_size.find(ptr);
   if (it != pool.block_size.end()) {
     const size_t block = it->second;
-    if (pool.enabled && pool.cached_bytes + block <= pool.limit_bytes) {
+    const bool keep = pool.enabled && pool.cached_bytes + block <= pool.limit_bytes;
+    auto slab = slab_of(pool, ptr);
+    if (slab != pool.slabs.end()) {
+      // Part of a slab: it waits on the free list, or the slab goes when this was its last block in use.
+      --slab->second.live;
+      if (!keep && slab->second.live == 0) {
+        pool_release_slab(pool, slab);
+      } else {
+        pool.free_blocks[block].push_back(ptr);
+        pool.cached_bytes += block;
+      }
+      return kOk;
+    }
+    if (keep) {
       pool.free_blocks[block].push_back(ptr);
       pool.cached_bytes += block;
       return kOk;
@@ -362,7 +453,7 @@ int ginn_hip_arena_create(ginn_hip_ctx* ctx, size_t bytes, ginn_hip_arena** aren
 int ginn_hip_arena_destroy(ginn_hip_arena* arena) {
   if (!arena) return kOk;
   (void)hipSetDevice(arena->ctx->device);
-  if (arena->base) (void)hipFree(arena->base);
+  if (arena->base) (void)ginn_hip_free(arena->ctx, arena->base);  // it came from ginn_hip_malloc
   delete arena;
   return kOk;
 }

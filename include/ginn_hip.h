@@ -113,7 +113,11 @@ int ginn_hip_sync(ginn_hip_ctx* ctx);
  * above) and handed out again without a driver call.  That is safe because a
  * context's memory is only used on its one stream: whatever still reads a
  * released block was enqueued before the block's next user.  Memory obtained
- * here must not be used on another stream without the caller's own ordering. */
+ * here must not be used on another stream without the caller's own ordering.
+ * Blocks of up to 64 KiB are cut, in address order, from 2 MiB driver
+ * allocations of their size class, which go back to the driver when none of
+ * their blocks is in use and the cache is emptied or over its bound: a graph
+ * of many small tensors costs few driver calls and its tensors share pages. */
 int ginn_hip_malloc(ginn_hip_ctx* ctx, size_t bytes, void** ptr);
 int ginn_hip_free(ginn_hip_ctx* ctx, void* ptr);
 /* The cache of released blocks: switch it off (enabled = 0: malloc / free go to
