@@ -117,7 +117,8 @@ __global__ __launch_bounds__(kBlock) void multi_apply_kernel(MultiParams p) {
 }
 
 // One record with the threads first, first + step, ... striding over it.
-__device__ __forceinline__ void apply_record(const ginn_hip_multi_op& op, size_t first, size_t step) {
+// By value: the caller reads a record from LDS in one go, not field by field.
+__device__ __forceinline__ void apply_record(const ginn_hip_multi_op op, size_t first, size_t step) {
   const OpKind k{op.kind, op.act, op.accumulate, op.value};
   switch (op.dtype) {
     case GINN_HIP_F32: apply_one<F32>(k, op.n, op.dst, op.src[0], op.src[1], op.src[2], first, step); break;
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(kBlock) void multi_mixed_kernel(const ginn_hip_mult
 // fetched into LDS once, and a stage of several short operations is dealt out
 // over the four waves (one operation per wave at a time) instead of running
 // them one after the other on the whole block.
-constexpr unsigned kChainLds = 96;      // records kept in LDS per batch
+constexpr unsigned kChainLds = 64;      // records kept in LDS per batch: one bit each in a 64-bit mask
 constexpr size_t kChainWaveOp = 4096;   // longest operation that one wave takes alone
 
 __global__ __launch_bounds__(kBlock) void multi_chain_kernel(const ginn_hip_multi_op* __restrict__ ops,
@@ -162,22 +163,25 @@ __global__ __launch_bounds__(kBlock) void multi_chain_kernel(const ginn_hip_mult
     uint4* dst = reinterpret_cast<uint4*>(recs);
     for (unsigned i = threadIdx.x; i < avail * kWords; i += kBlock) dst[i] = src[i];
     __syncthreads();
+    // Where the stages begin and which records are long, one bit per record, found by every wave
+    // for itself (two LDS reads): the stage loop below then reads nothing.  (Scanning the records
+    // for the end of each stage cost more than the stages' arithmetic.)
+    const bool present = lane < avail;
+    const bool begin = present && (lane == 0 || recs[lane].reserved != recs[lane - 1].reserved);
+    const unsigned long long begins = __ballot(begin);
+    const unsigned long long longs = __ballot(present && recs[lane].n > kChainWaveOp);
     unsigned take = avail;
     if (base + avail < c.count) {
-      const int last = recs[avail - 1].reserved;
-      unsigned cut = avail;
-      while (cut > 0 && recs[cut - 1].reserved == last) --cut;
+      const unsigned cut = 63u - static_cast<unsigned>(__builtin_clzll(begins));  // bit 0 is set
       if (cut > 0) take = cut;  // leave the unfinished stage to the next batch
     }
     unsigned i = 0;
     while (i < take) {
-      unsigned j = i;
-      size_t longest = 0;
-      while (j < take && recs[j].reserved == recs[i].reserved) {
-        longest = max(longest, recs[j].n);
-        ++j;
-      }
-      if (j - i >= 2 && longest <= kChainWaveOp) {
+      const unsigned long long later = i + 1 < 64 ? begins >> (i + 1) : 0ull;
+      unsigned j = later ? i + 1 + static_cast<unsigned>(__builtin_ctzll(later)) : take;
+      if (j > take) j = take;
+      const unsigned long long stage = (j - i < 64 ? (1ull << (j - i)) - 1 : ~0ull) << i;
+      if (j - i >= 2 && !(longs & stage)) {
         for (unsigned r = i + wave; r < j; r += kBlock / 64) apply_record(recs[r], lane, 64);
       } else {
         for (unsigned r = i; r < j; ++r) apply_record(recs[r], threadIdx.x, kBlock);
