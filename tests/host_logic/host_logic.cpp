@@ -96,6 +96,34 @@ int main() {
   g.backward(1.);
   report("plain pass");
 
+  // A leaf whose gradient gets a reduction on two levels (a bias added in two layers, five
+  // columns each): level by level these are two reductions of five sources; a frozen executor
+  // sums all ten at the end of the backward pass.
+  {
+    auto bias = Random(dev, {8});
+    bias->set_has_grad(true);
+    std::vector<NodePtr<Real>> tops;
+    for (int i = 0; i < 5; ++i) {
+      auto xi = Random(dev, {8});
+      auto lower = Add(NodePtr<Real>(xi), NodePtr<Real>(bias));
+      tops.push_back(Add(NodePtr<Real>(Tanh(NodePtr<Real>(lower))), NodePtr<Real>(bias)));
+    }
+    Graph two(Sum(NodePtr<Real>(Add(tops))));
+    LevelExecutor ex2(two);
+    ex2.reset_forwarded();
+    ex2.forward();
+    ex2.reset_grad();
+    null_abi_clear();
+    ex2.backward(1.);
+    report("two-level backward");
+    ex2.freeze();
+    ex2.forward();
+    ex2.reset_grad();
+    null_abi_clear();
+    ex2.backward(1.);
+    report("two-level backward frozen");
+  }
+
   // Autobatch (ginn/autobatch.h:42-202): six Affines that share W on one
   // height and two that share it on the next become two merged products.
   {

@@ -7,7 +7,8 @@ table launches every phase made.  Checked here: one launch per level whatever
 the nodes compute, one zero fill for all gradients, a reduction for five users
 of one gradient, successive launches for two users of one gradient on one
 level, plans reused without uploads on the second pass, the frozen replay
-making the same launches, and plain execution making none of them.
+making the same launches (and one reduction per pass into a leaf's gradient instead of one per
+level), and plain execution making none of them.
 """
 import re
 import subprocess
@@ -102,6 +103,17 @@ def test_fused_levels_become_chain_launches(phases):
     assert bcalls == [("multi_mixed", 2), ("multi_chain", 1), ("multi_reduce", 5), ("multi_mixed", 3),
                       ("multi_chain", 2)]
     assert int(phases["chain launches built"]) == 3
+
+
+def test_frozen_pass_sums_a_leaf_gradient_once(phases):
+    """Two levels each add five gradients into one bias: a reduction per level while every node is
+    asked, ONE reduction over all ten sources at the end of a frozen backward pass."""
+    calls, _, _ = phases["two-level backward"]
+    assert calls.count(("multi_reduce", 5)) == 2
+    frozen, uploads, _ = phases["two-level backward frozen"]
+    assert [c for c in frozen if c[0] == "multi_reduce"] == [("multi_reduce", 10)]
+    assert frozen[-1] == ("multi_reduce", 10) and uploads == 0
+    assert [c for c in frozen if c[0] != "multi_reduce"] == [c for c in calls if c[0] != "multi_reduce"]
 
 
 def test_plain_execution_launches_per_node(phases):
