@@ -132,6 +132,7 @@ PROTOTYPES = {
                                      c_void_p, c_void_p, c_void_p]),
     "ginn_hip_multi_mixed": (c_int, [c_void_p, c_int, c_void_p, c_size_t]),
     "ginn_hip_multi_chain": (c_int, [c_void_p, c_int, c_void_p, c_void_p]),
+    "ginn_hip_ctx_wait_for": (c_int, [c_void_p, c_void_p, POINTER(c_int)]),
     "ginn_hip_multi_reduce": (c_int, [c_void_p, c_int, c_size_t, c_int, c_void_p, c_void_p, c_int]),
     "ginn_hip_multi_zero": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_size_t]),
     "ginn_hip_update": (c_int, [c_void_p, c_void_p, c_int, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p]),

@@ -104,6 +104,7 @@ struct ginn_hip_ctx {
   size_t host_staging_bytes = 0;
   size_t host_staging_used = 0;  // ring cursor
   hipEvent_t staging_event = nullptr;
+  hipEvent_t order_event = nullptr;  // ginn_hip_ctx_wait_for with this context as the signaler
   std::mutex mutex;  // serialises workspace users across host threads
   hipEvent_t events[64] = {};
   int num_cus = 256;

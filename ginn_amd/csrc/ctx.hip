@@ -4,6 +4,7 @@
 #include <string>
 
 #include <algorithm>
+#include <cstdlib>
 #include <iterator>
 
 #include "common.h"
@@ -231,6 +232,7 @@ int ginn_hip_ctx_destroy(ginn_hip_ctx* ctx) {
   for (auto& ev : ctx->events)
     if (ev) (void)hipEventDestroy(ev);
   if (ctx->staging_event) (void)hipEventDestroy(ctx->staging_event);
+  if (ctx->order_event) (void)hipEventDestroy(ctx->order_event);
   if (ctx->host_staging) (void)hipHostFree(ctx->host_staging);
   if (ctx->workspace) (void)hipFree(ctx->workspace);
   if (ctx->folds.arena) (void)hipFree(ctx->folds.arena);
@@ -498,6 +500,32 @@ int ginn_hip_arena_used(const ginn_hip_arena* arena, size_t* bytes) {
 int ginn_hip_arena_size(const ginn_hip_arena* arena, size_t* bytes) {
   GH_CHECK_ARG(arena && bytes, "ginn_hip_arena_size: NULL argument");
   *bytes = arena->size;
+  return kOk;
+}
+
+int ginn_hip_ctx_wait_for(ginn_hip_ctx* waiter, ginn_hip_ctx* signaler, int* ordered) {
+  GH_CHECK_ARG(waiter && signaler && ordered, "ginn_hip_ctx_wait_for: NULL argument");
+  GH_CHECK_ARG(waiter->device == signaler->device, "ginn_hip_ctx_wait_for: contexts of devices %d and %d",
+               waiter->device, signaler->device);
+  *ordered = 0;
+  if (waiter == signaler || waiter->stream == signaler->stream) {
+    *ordered = 1;  // one stream: already in order
+    return kOk;
+  }
+  GH_HIP(hipSetDevice(signaler->device));
+  for (ginn_hip_ctx* c : {waiter, signaler}) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    GH_HIP(hipStreamIsCapturing(c->stream, &status));
+    if (status != hipStreamCaptureStatusNone) return kOk;
+  }
+  {
+    std::lock_guard<std::mutex> lock(signaler->mutex);
+    if (!signaler->order_event) GH_HIP(hipEventCreateWithFlags(&signaler->order_event, hipEventDisableTiming));
+    // The wait below refers to this record; a later record by another host thread does not change it.
+    GH_HIP(hipEventRecord(signaler->order_event, signaler->stream));
+    GH_HIP(hipStreamWaitEvent(waiter->stream, signaler->order_event, 0));
+  }
+  *ordered = 1;
   return kOk;
 }
 

@@ -14,6 +14,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -119,15 +120,26 @@ namespace internal {
 // any static destructor of this header would run.
 class ContextTable {
   std::vector<ginn_hip_ctx*> ctx_;
+  // A second context (stream, workspace) per GPU for work that nothing on the
+  // first one's stream waits for (ginn_hip_ctx_wait_for); no memory of tensors
+  // is ever allocated on it.
+  std::vector<ginn_hip_ctx*> beside_;
+  std::mutex mutex_;
 
  public:
-  ContextTable() : ctx_(static_cast<size_t>(std::max(gpus(), 0)), nullptr) {}
+  ContextTable() : ctx_(static_cast<size_t>(std::max(gpus(), 0)), nullptr), beside_(ctx_.size(), nullptr) {}
   ContextTable(const ContextTable&) = delete;
   ginn_hip_ctx*& at(size_t idx) {
     GINN_ASSERT(idx < ctx_.size(),
                 "no GPU with index " + std::to_string(idx) + " (" + std::to_string(ctx_.size()) + " visible)");
     if (!ctx_[idx]) GINN_HIP_CALL(ginn_hip_ctx_create(static_cast<int>(idx), 0, &ctx_[idx]));
     return ctx_[idx];
+  }
+  ginn_hip_ctx* beside(size_t idx) {
+    GINN_ASSERT(idx < beside_.size());
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (!beside_[idx]) GINN_HIP_CALL(ginn_hip_ctx_create(static_cast<int>(idx), 0, &beside_[idx]));
+    return beside_[idx];
   }
 };
 inline ContextTable& contexts() {

@@ -351,9 +351,12 @@ class FoldWindow {
     auto& v = touched();
     if (std::find(v.begin(), v.end(), ctx) == v.end()) v.push_back(ctx);
   }
-  static void at_close(void (*fn)(int)) {
+  // first: ahead of the hooks registered so far (work that the others' work must find finished).
+  static void at_close(void (*fn)(int), bool first = false) {
     auto& v = hooks();
-    if (std::find(v.begin(), v.end(), fn) == v.end()) v.push_back(fn);
+    if (std::find(v.begin(), v.end(), fn) != v.end()) return;
+    if (first) v.insert(v.begin(), fn);
+    else v.push_back(fn);
   }
   // The end of the pass: the outermost window folds what was postponed.
   void close() {
@@ -371,6 +374,47 @@ class FoldWindow {
     std::vector<ginn_hip_ctx*> v;
     v.swap(touched());
     for (ginn_hip_ctx* c : v) GINN_HIP_CALL(ginn_hip_flush_folds(c));
+  }
+};
+
+// Products into the gradients of leaves (weights) beside the pass.  Every other product of a
+// backward pass feeds the next node, one launch after the other, and many of them leave a
+// quarter to a half of the CUs idle (144 or 192 tiles on 256 CUs); the gradient of a weight is
+// needed by nobody until the pass ends.  While a pass runs, such a product is therefore enqueued
+// on the GPU's second context: its stream waits for what the pass has enqueued so far (the
+// product's operands), the pass goes on without waiting for it, and the end of the pass waits for
+// the second stream.  The operands are a node's gradient and another node's value (or a buffer
+// the node keeps), none of which changes before the next pass.  Same kernels, same results.
+class BesidePass {
+  static std::vector<std::pair<ginn_hip_ctx*, ginn_hip_ctx*>>& joined() {
+    thread_local std::vector<std::pair<ginn_hip_ctx*, ginn_hip_ctx*>> v;  // (main, beside) used in this pass
+    return v;
+  }
+  static void join(int) {  // also when the pass ends by an exception
+    std::vector<std::pair<ginn_hip_ctx*, ginn_hip_ctx*>> v;
+    v.swap(joined());
+    for (auto& [main, beside] : v) {
+      int ordered = 0;
+      (void)ginn_hip_ctx_wait_for(main, beside, &ordered);
+      if (!ordered) (void)ginn_hip_sync(beside);  // cannot happen: no capture began since the product
+    }
+  }
+
+ public:
+  static constexpr double kWorthIt = 1e9;  // flops below which the two events cost more than the overlap gains
+  // The context to enqueue a product of `flops` into the gradient of `target` on.
+  static ginn_hip_ctx* ctx_for(const BaseNode& target, const DevPtr& dev, double flops) {
+    const size_t idx = dev->id().idx;
+    ginn_hip_ctx* main = contexts().at(idx);
+    if (!FoldWindow::open() || !target.inputs().empty() || flops < kWorthIt) return main;
+    ginn_hip_ctx* beside = contexts().beside(idx);
+    int ordered = 0;
+    GINN_HIP_CALL(ginn_hip_ctx_wait_for(beside, main, &ordered));
+    if (!ordered) return main;  // a device graph is being recorded: one stream
+    auto& v = joined();
+    if (std::find(v.begin(), v.end(), std::make_pair(main, beside)) == v.end()) v.emplace_back(main, beside);
+    FoldWindow::at_close(&join, /*first=*/true);
+    return beside;
   }
 };
 

@@ -72,15 +72,24 @@ class AffineNode : public BaseDataNode<Scalar> {
                                           value().data(), preactiv_.size() > 0 ? preactiv_.data() : nullptr,
                                           identity ? nullptr : dpreactiv_.data(),
                                           bias->has_grad() ? bias->grad().data() : nullptr));
-    for (size_t i = 0; i + 1 < ins_.size(); i += 2) {
-      auto &a = ins_[i], &b = ins_[i + 1];
-      if (b->has_grad()) {
-        const bool fresh = b->take_lazy_zero();
-        gpu_prod(b->grad(), a->value(), daffine, fresh ? ProdResult::Assign : ProdResult::Add, ProdTranspose::First);
-      }
-      if (a->has_grad()) {
-        const bool fresh = a->take_lazy_zero();
-        gpu_prod(a->grad(), daffine, b->value(), fresh ? ProdResult::Assign : ProdResult::Add, ProdTranspose::Second);
+    // The gradients the nodes below wait for first; those of leaves (weights) beside the pass:
+    // daffine is this node's gradient or a buffer it keeps, unchanged until the next pass.
+    for (const bool leaves : {false, true}) {
+      for (size_t i = 0; i + 1 < ins_.size(); i += 2) {
+        auto &a = ins_[i], &b = ins_[i + 1];
+        const double flops = 2.0 * static_cast<double>(m) * static_cast<double>(n) * static_cast<double>(a->value().cols());
+        if (b->has_grad() && b->inputs().empty() == leaves) {
+          const bool fresh = b->take_lazy_zero();
+          ginn_hip_ctx* where = BesidePass::ctx_for(*b, dev(), flops);
+          gpu_prod(where, b->grad(), a->value(), daffine, fresh ? ProdResult::Assign : ProdResult::Add,
+                   ProdTranspose::First);
+        }
+        if (a->has_grad() && a->inputs().empty() == leaves) {
+          const bool fresh = a->take_lazy_zero();
+          ginn_hip_ctx* where = BesidePass::ctx_for(*a, dev(), flops);
+          gpu_prod(where, a->grad(), daffine, b->value(), fresh ? ProdResult::Assign : ProdResult::Add,
+                   ProdTranspose::Second);
+        }
       }
     }
   }

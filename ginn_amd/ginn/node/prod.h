@@ -24,13 +24,21 @@ class ProdNode : public BaseDataNode<Scalar> {
   }
   void backward_() override {
     using namespace internal;
-    if (b_->has_grad()) {
-      const bool fresh = b_->take_lazy_zero();
-      gpu_prod(b_->grad(), a_->value(), grad(), fresh ? ProdResult::Assign : ProdResult::Add, ProdTranspose::First);
-    }
-    if (a_->has_grad()) {
-      const bool fresh = a_->take_lazy_zero();
-      gpu_prod(a_->grad(), grad(), b_->value(), fresh ? ProdResult::Assign : ProdResult::Add, ProdTranspose::Second);
+    // A gradient that is a leaf's (a weight's) is formed beside the pass, the other one first.
+    const double flops = 2.0 * static_cast<double>(grad().size()) * static_cast<double>(a_->value().cols());
+    for (const bool leaves : {false, true}) {
+      if (b_->has_grad() && b_->inputs().empty() == leaves) {
+        const bool fresh = b_->take_lazy_zero();
+        ginn_hip_ctx* where = BesidePass::ctx_for(*b_, dev(), flops);
+        gpu_prod(where, b_->grad(), a_->value(), grad(), fresh ? ProdResult::Assign : ProdResult::Add,
+                 ProdTranspose::First);
+      }
+      if (a_->has_grad() && a_->inputs().empty() == leaves) {
+        const bool fresh = a_->take_lazy_zero();
+        ginn_hip_ctx* where = BesidePass::ctx_for(*a_, dev(), flops);
+        gpu_prod(where, a_->grad(), grad(), b_->value(), fresh ? ProdResult::Assign : ProdResult::Add,
+                 ProdTranspose::Second);
+      }
     }
   }
 

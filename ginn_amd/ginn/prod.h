@@ -48,8 +48,9 @@ enum class ProdResult { Assign, Add };
 enum class ProdTranspose { None, First, Second, Both };
 
 // c (+)= op(a) * op(b) on the rank-2 folds of the tensors (ginn/prod.h:211-253).
+// The first form runs on the context given (internal::BesidePass), the second on the context of c's GPU.
 template <typename Scalar>
-inline void gpu_prod(Tensor<Scalar>& c, Tensor<Scalar>& a, Tensor<Scalar>& b,
+inline void gpu_prod(ginn_hip_ctx*& handle, Tensor<Scalar>& c, Tensor<Scalar>& a, Tensor<Scalar>& b,
                      ProdResult res = ProdResult::Assign, ProdTranspose tra = ProdTranspose::None) {
   const bool ta = tra == ProdTranspose::First || tra == ProdTranspose::Both;
   const bool tb = tra == ProdTranspose::Second || tra == ProdTranspose::Both;
@@ -60,11 +61,16 @@ inline void gpu_prod(Tensor<Scalar>& c, Tensor<Scalar>& a, Tensor<Scalar>& b,
   GINN_ASSERT(a_outer == c.rows());
   GINN_ASSERT(b_outer == c.cols());
 
-  gpu_gemm<Scalar>(cublas_handle(static_cast<int>(c.dev()->id().idx)), a.data(), b.data(), c.data(),
+  gpu_gemm<Scalar>(handle, a.data(), b.data(), c.data(),
                    /* lda */ static_cast<int>(a.rows()), /* ldb */ static_cast<int>(b.rows()),
                    /* ldc */ static_cast<int>(c.rows()), /* m */ static_cast<int>(a_outer),
                    /* k */ static_cast<int>(a_inner), /* n */ static_cast<int>(b_outer),
                    res == ProdResult::Add ? Scalar(1.f) : Scalar(0.f), ta ? OP_T : OP_N, tb ? OP_T : OP_N);
+}
+template <typename Scalar>
+inline void gpu_prod(Tensor<Scalar>& c, Tensor<Scalar>& a, Tensor<Scalar>& b,
+                     ProdResult res = ProdResult::Assign, ProdTranspose tra = ProdTranspose::None) {
+  gpu_prod(cublas_handle(static_cast<int>(c.dev()->id().idx)), c, a, b, res, tra);
 }
 
 // c[:, :, i] (+)= op(a[:, :, i]) * op(b[:, :, i]) on the rank-3 folds

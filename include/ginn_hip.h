@@ -99,6 +99,22 @@ int ginn_hip_ctx_destroy(ginn_hip_ctx* ctx);
 int ginn_hip_ctx_device(const ginn_hip_ctx* ctx, int* device);
 int ginn_hip_ctx_stream(const ginn_hip_ctx* ctx, void** stream);
 
+/* Orders two contexts of one device: what is enqueued on `waiter` after this
+ * call runs after everything enqueued on `signaler` before it (an event
+ * recorded on one stream and waited for on the other; the host does not
+ * wait).  With it work that nothing on a context's stream depends on can run
+ * beside that stream on a second context and be joined later: the drop-in
+ * headers run the products into the gradients of weights (leaves, complete
+ * only when the backward pass ends: ginn/node/prod.h:57-63,
+ * ginn/node/affine.h:117-122) that way, so they share the device with the
+ * chain of launches every other node waits for instead of each taking its
+ * turn with a part of it.  The reference has one handle and the legacy
+ * default stream (ginn/dev.h:188-189).  *ordered is set to 0, and nothing is
+ * enqueued, while either stream is recording a device graph: the caller then
+ * keeps the work on one context. */
+int ginn_hip_ctx_wait_for(ginn_hip_ctx* waiter, ginn_hip_ctx* signaler,
+                          int* ordered);
+
 /* Blocks until the context's stream is idle (cudaStreamSynchronize /
  * cudaDeviceSynchronize as used in ginn/util/timer.h:36-45). */
 int ginn_hip_sync(ginn_hip_ctx* ctx);

@@ -106,3 +106,45 @@ def test_arena_is_byte_exact_and_fills_work_at_any_alignment(ctx):
     lib.call("ginn_hip_arena_used", arena, byref(used))
     assert p2.value == p1.value + 64 and used.value == 67
     lib.call("ginn_hip_arena_destroy", arena)
+
+
+def test_a_context_waits_for_another(ctx):
+    """ginn_hip_ctx_wait_for: what is enqueued on the waiter afterwards sees everything the signaler had
+    enqueued before (no host wait in between); one stream needs no event; while a device graph is being
+    recorded nothing is ordered and the caller is told so."""
+    from ctypes import c_int
+    lib, a = ctx
+    b = lib.ctx_create(0)
+    try:
+        n = 1 << 24
+        buf, out = c_void_p(), c_void_p()
+        lib.call("ginn_hip_malloc", a, 4 * n, byref(buf))
+        lib.call("ginn_hip_malloc", a, 4 * n, byref(out))
+        lib.call("ginn_hip_fill", a, capi.F32, out, n, -1.0)
+        lib.call("ginn_hip_sync", a)
+        for i in range(40):  # a queue of fills on a; the last one counts
+            lib.call("ginn_hip_fill", a, capi.F32, buf, n, float(i))
+        ordered = c_int(-1)
+        lib.call("ginn_hip_ctx_wait_for", b, a, byref(ordered))
+        assert ordered.value == 1
+        lib.call("ginn_hip_memcpy_d2d", b, out, buf, 4 * n)
+        host = np.zeros(n, np.float32)
+        lib.call("ginn_hip_memcpy_d2h", b, host.ctypes.data_as(c_void_p), out, 4 * n)
+        assert (host == 39.0).all()
+        lib.call("ginn_hip_ctx_wait_for", a, a, byref(ordered))
+        assert ordered.value == 1
+        lib.call("ginn_hip_capture_begin", a)
+        try:
+            lib.call("ginn_hip_fill", a, capi.F32, buf, n, 5.0)
+            lib.call("ginn_hip_ctx_wait_for", b, a, byref(ordered))
+            assert ordered.value == 0
+        finally:
+            graph = c_void_p()
+            lib.call("ginn_hip_capture_end", a, byref(graph))
+            lib.call("ginn_hip_graph_destroy", graph)
+        with pytest.raises(capi.GinnHipError, match="NULL"):
+            lib.call("ginn_hip_ctx_wait_for", b, None, byref(ordered))
+        lib.call("ginn_hip_free", a, buf)
+        lib.call("ginn_hip_free", a, out)
+    finally:
+        lib.call("ginn_hip_ctx_destroy", b)
