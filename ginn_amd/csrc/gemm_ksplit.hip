@@ -5,9 +5,11 @@
 // most.  Tiles of 64 x 64 with K split over workgroups fill the machine but
 // need a second launch that folds the partial sums, which costs as much as
 // the product itself (4 us against 7).  Here a workgroup of 16 waves owns one
-// 32 x 32 tile, every wave walks one sixteenth of K with operands straight
-// from memory in the matrix instruction's own layout (no staging, no barrier
-// in the loop), and the 16 partial tiles meet in LDS, always in the same order.
+// 32 x 32 tile and every wave walks one sixteenth of K on its own, without a
+// barrier in the loop: an operand whose rows are contiguous in memory arrives
+// in the matrix instruction's layout as it is loaded, a K-contiguous one is
+// turned through a slice of LDS that belongs to the wave.  The 16 partial
+// tiles meet in LDS and are added in wave order.
 #include "common.h"
 
 namespace ginn_hip {
