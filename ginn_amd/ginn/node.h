@@ -385,6 +385,10 @@ class FoldWindow {
 // product's operands), the pass goes on without waiting for it, and the end of the pass waits for
 // the second stream.  The operands are a node's gradient and another node's value (or a buffer
 // the node keeps), none of which changes before the next pass.  Same kernels, same results.
+inline bool& beside_pass_flag() {
+  static bool on = true;
+  return on;
+}
 class BesidePass {
   static std::vector<std::pair<ginn_hip_ctx*, ginn_hip_ctx*>>& joined() {
     thread_local std::vector<std::pair<ginn_hip_ctx*, ginn_hip_ctx*>> v;  // (main, beside) used in this pass
@@ -406,7 +410,7 @@ class BesidePass {
   static ginn_hip_ctx* ctx_for(const BaseNode& target, const DevPtr& dev, double flops) {
     const size_t idx = dev->id().idx;
     ginn_hip_ctx* main = contexts().at(idx);
-    if (!FoldWindow::open() || !target.inputs().empty() || flops < kWorthIt) return main;
+    if (!beside_pass_flag() || !FoldWindow::open() || !target.inputs().empty() || flops < kWorthIt) return main;
     ginn_hip_ctx* beside = contexts().beside(idx);
     int ordered = 0;
     GINN_HIP_CALL(ginn_hip_ctx_wait_for(beside, main, &ordered));
@@ -445,6 +449,11 @@ inline std::vector<BaseNode*>*& lazy_take_log() {
   return log;
 }
 }  // namespace internal
+
+// Whether products into the gradients of weights may run on the GPU's second stream while a
+// backward pass runs (internal::BesidePass); on by default.
+inline void set_beside_pass(bool on) { internal::beside_pass_flag() = on; }
+inline bool beside_pass() { return internal::beside_pass_flag(); }
 
 // Whether reset_grad() of Graph and LevelExecutor may flag gradients instead of
 // zeroing them (BaseNode::GradUse); on by default.

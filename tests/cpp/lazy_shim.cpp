@@ -155,6 +155,9 @@ int shim_lazy_graph(int dtype, int lazy, int mode, int passes, int hs, int nh, i
                                  out_flagged, out_fills)));
 }
 
+// Products into weight gradients on the second stream of the GPU (on by default) or on the one stream.
+void shim_set_beside_pass(int on) { set_beside_pass(on != 0); }
+
 // What everybody but the one overwriting user sees of a flagged gradient.
 // which: 0 = read between reset_grad() and backward(): zeros, not what the
 // last pass left; 1 = two graphs that share a node, reset one after the other

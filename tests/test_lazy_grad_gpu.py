@@ -117,3 +117,25 @@ def test_only_single_overwriting_users_qualify(shim):
     # A, B (Prod overwrites), Sum(P) and Sum(Q) (Add overwrites); not P (three
     # uses), not Q (Sum adds to its input), not the sink.
     assert out[0] == 4
+
+
+@pytest.mark.parametrize("dt", [capi.F32, capi.BF16])
+@pytest.mark.parametrize("mode", ["graph", "executor", "frozen", "recorded"])
+def test_weight_gradients_beside_the_pass_are_the_same_bits(shim, dt, mode):
+    """Products of >= 1 GFLOP into the gradients of weights run on the GPU's second stream while a
+    backward pass runs (internal::BesidePass in ginn_amd/ginn/node.h; the reference has one stream,
+    ginn/dev.h:188-189).  Same kernels on the same operands: after three passes without a wait in
+    between, loss and every gradient are bit-identical to the run on one stream."""
+    sizes = dict(hs=64, nh=12, B=4, T=256, V=1024)  # 768 x 768 x 1024 products: 1.2 GFLOP each
+    try:
+        shim.shim_set_beside_pass(0)
+        want_loss, want_dx, want_grads, _, _ = run(shim, dt, 1, mode, 3, seed=11, **sizes)
+        shim.shim_set_beside_pass(1)
+        got_loss, got_dx, got_grads, _, _ = run(shim, dt, 1, mode, 3, seed=11, **sizes)
+    finally:
+        shim.shim_set_beside_pass(1)
+    assert got_loss == want_loss
+    np.testing.assert_array_equal(got_dx, want_dx)
+    for g, w in zip(got_grads, want_grads):
+        assert np.abs(w).max() > 0
+        np.testing.assert_array_equal(g, w)
