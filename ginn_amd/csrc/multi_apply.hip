@@ -79,6 +79,30 @@ __device__ __forceinline__ void apply_one(const OpKind& k, size_t n, void* dst_,
   const bool has1 = s1 != nullptr, has2 = s2 != nullptr;
   const uintptr_t bits = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(s0) |
                          reinterpret_cast<uintptr_t>(s1) | reinterpret_cast<uintptr_t>(s2);
+  if constexpr (sizeof(S) == 4) {
+    // fp32, a short operation (one pass of the lanes covers it): four elements per lane instead of eight.
+    // What such an operation costs is the length of the dependent instruction stream of one wave, and the
+    // transcendental functions of fp32 are long: with four elements the wave issues half as many
+    // instructions, still with four independent chains to fill the pipeline (one element per lane was
+    // measured too: no better), and the access is one 16-byte vector per operand either way.
+    if (bits % 16 == 0 && n % 4 == 0 && n <= 4 * step) {
+      const size_t i = first * 4;
+      if (i < n) {
+        float a[4], b[4], c[4], d[4], v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[e] = b[e] = c[e] = d[e] = 0.f;
+        if (s0) ld<T, 4>(s0 + i, a);
+        if (has1) ld<T, 4>(s1 + i, b);
+        if (has2) ld<T, 4>(s2 + i, c);
+        if (k.accumulate) ld<T, 4>(dst + i, d);
+        multi_values<FAST, 4>(k, a, b, c, v);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += d[e];
+        st<T, 4>(dst + i, v);
+      }
+      return;
+    }
+  }
   if (bits % 16 == 0 && n % 8 == 0) {
     for (size_t i = first * 8; i < n; i += step * 8) {
       float a[8], b[8], c[8], d[8], v[8];

@@ -16,6 +16,10 @@ template <typename T, int V>
 __device__ __forceinline__ void ld(const typename T::storage* p, float (&v)[V]) {
   if constexpr (V == 1) {
     v[0] = to_float<T>(p[0]);
+  } else if constexpr (sizeof(typename T::storage) == 4 && V == 4) {
+    const va_f32x4 q = *reinterpret_cast<const va_f32x4*>(p);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = q[e];
   } else if constexpr (sizeof(typename T::storage) == 4) {
     static_assert(V == 8, "vector width is 8");
     const va_f32x4 lo = *reinterpret_cast<const va_f32x4*>(p);
@@ -40,6 +44,8 @@ template <typename T, int V>
 __device__ __forceinline__ void st(typename T::storage* p, const float (&v)[V]) {
   if constexpr (V == 1) {
     p[0] = from_float<T>(v[0]);
+  } else if constexpr (sizeof(typename T::storage) == 4 && V == 4) {
+    *reinterpret_cast<va_f32x4*>(p) = va_f32x4{v[0], v[1], v[2], v[3]};
   } else if constexpr (sizeof(typename T::storage) == 4) {
     va_f32x4 lo, hi;
 #pragma unroll
