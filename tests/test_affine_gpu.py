@@ -304,7 +304,8 @@ def _scatter_columns(dev, M, dt, rng, misalign=False):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("m,k,n", [(96, 72, 40), (64, 64, 64), (130, 33, 7), (1024, 384, 200), (8, 8, 1)])
+@pytest.mark.parametrize("m,k,n", [(96, 72, 40), (64, 64, 64), (130, 33, 7), (1024, 384, 200), (8, 8, 1),
+                                   (1024, 384, 100)])  # fp32: the scattered dX on 16 x 16 tiles
 @pytest.mark.parametrize("misalign", [False, True])
 def test_gathered_gemm(dev, dt, m, k, n, misalign):
     """The three products of a merged Autobatch group on operands that stay
@@ -354,7 +355,8 @@ def test_gathered_gemm(dev, dt, m, k, n, misalign):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("m,n,k", [(96, 72, 40), (64, 64, 300), (130, 33, 7), (1024, 384, 1500), (8, 12, 1), (5, 3, 0)])
+@pytest.mark.parametrize("m,n,k", [(96, 72, 40), (64, 64, 300), (130, 33, 7), (1024, 384, 1500), (8, 12, 1), (5, 3, 0),
+                                   (96, 72, 600), (50, 19, 1024)])  # fp32: both tables on 16 x 16 tiles
 @pytest.mark.parametrize("misalign", [False, True])
 @pytest.mark.parametrize("beta", [0.0, 1.0])
 def test_outer_sum_of_scattered_columns(dev, dt, m, n, k, misalign, beta):

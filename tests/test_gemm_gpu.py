@@ -76,7 +76,9 @@ def test_reference_prod_golden(dev, golden, dt, op_a, op_b):
                                    # fp32: one launch with K split inside the workgroup, up to its limits
                                    # (256 tiles of 32 x 32, K = 1024) and just beyond
                                    (33, 31, 36), (1024, 256, 384), (384, 250, 1024), (500, 500, 1000),
-                                   (96, 40, 1028)])
+                                   (96, 40, 1028),
+                                   # ... on 16 x 16 tiles (few large tiles, a long sum), ragged edges
+                                   (384, 120, 1024), (50, 19, 520), (17, 250, 1000)])
 @pytest.mark.parametrize("beta", [0.0, 1.0])
 def test_small_shapes(dev, dt, op_a, op_b, m, n, k, beta):
     run_case(dev, dt, op_a, op_b, m, n, k, beta, seed=m * 7 + n * 3 + k)
