@@ -315,10 +315,12 @@ int launch_gemm_ksplit(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (akc && !aligned(a.A, a.lda)) return kUnsupported;
   if (bkc && !(a.bcols ? a.cols_vec_ld : aligned(a.B, a.ldb))) return kUnsupported;
   // Few 32 x 32 tiles with a long sum: 16 x 16 tiles put four times as many CUs to work (see Shape),
-  // and read the operands twice as often: beyond one tile per CU that costs more than it gains
-  // (384 x 256 x 1024: 9.7 us on 384 small tiles, 8.8 us on 96 large ones).
+  // and read the operands twice as often.  Measured where that stops to pay: with a row-contiguous A
+  // two small tiles per CU are still ahead (512 x 256 x 1024: 7.9 us on 512 small tiles, 9.5 us on
+  // 128 large ones), with both operands K-contiguous one per CU is the limit (384 x 256 x 1024:
+  // 9.7 us on 384 small tiles, 8.8 us on 96 large ones).
   const long long small_tiles = static_cast<long long>((a.m + 15) / 16) * ((a.n + 15) / 16);
-  if (tiles * 2 <= ctx->num_cus && a.k >= 512 && small_tiles <= ctx->num_cus)
+  if (tiles * 2 <= ctx->num_cus && a.k >= 256 && small_tiles <= (akc ? 1 : 2) * static_cast<long long>(ctx->num_cus))
     return launch_tile<16>(ctx, p, akc, bkc);
   return launch_tile<32>(ctx, p, akc, bkc);
 }
