@@ -234,7 +234,7 @@ __global__ __launch_bounds__(kThreadsB) void gemm_bsmall_kernel(Params p) {
   for (int it = 0; it < 32 * FN / kColsPerIter; ++it) {
     const int col = it * kColsPerIter + sub;
     const u32x4 v = *reinterpret_cast<const u32x4*>(stage + col * G::kEpiColStride + chunk * 16);
-    *reinterpret_cast<u32x4*>(C + (long long)(n0 + wn + col) * p.ldc + m0 + wm + chunk * 8) = v;
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (long long)(n0 + wn + col) * p.ldc + m0 + wm + chunk * 8));
   }
 }
 
