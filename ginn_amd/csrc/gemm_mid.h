@@ -706,6 +706,7 @@ int launch_shape(ginn_hip_ctx* ctx, const MidParams& p, int dtype, int batch, in
 extern template int launch_shape<2, 2>(ginn_hip_ctx*, const MidParams&, int, int, int, int, bool, bool);
 extern template int launch_shape<2, 1>(ginn_hip_ctx*, const MidParams&, int, int, int, int, bool, bool);
 extern template int launch_shape<1, 2>(ginn_hip_ctx*, const MidParams&, int, int, int, int, bool, bool);
+extern template int launch_shape<1, 1>(ginn_hip_ctx*, const MidParams&, int, int, int, int, bool, bool);
 
 }  // namespace mid
 }  // namespace ginn_hip

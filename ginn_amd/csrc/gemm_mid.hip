@@ -39,18 +39,38 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
   // until about every CU has a workgroup; if that still leaves most of the
   // chip idle the generic kernel's 64 x 64 tiles do better.
   const bool f32 = a.dtype == GINN_HIP_F32;
-  bool f32_small = false;
+  bool f32_small = false, f32_tiny_tiles = false;
   if (f32) {
     const long long tiles128 = (long long)((a.m + 127) / 128) * ((a.n + 127) / 128) * a.batch;
     if (tiles128 * 2 < ctx->num_cus) {
       f32_small = true;
-      if (fm == 2 && fn == 2) fn = 1;
+      // 64 x 64 tiles when they give most CUs a workgroup without a K split:
+      // the same matrix-pipe time per CU as 128 x 64 tiles over half of K each,
+      // and no partial tiles to fold in a second launch (which costs what
+      // some 20 K tiles of such a workgroup cost: the fewer the tiles, the
+      // shorter the K up to which that holds).
+      const long long tiles64 = (long long)(a.m / 64) * (a.n / 64) * a.batch;
+      const int kt = a.k / bk;
+      const bool enough = tiles64 >= ctx->num_cus || (tiles64 * 4 >= 3 * ctx->num_cus && kt <= 64) ||
+                          (tiles64 * 8 >= 3 * ctx->num_cus && kt <= 32);
+      if (a.m % 64 == 0 && a.n % 64 == 0 && enough && tiles64 <= 2 * ctx->num_cus)
+        fm = 1, fn = 1, f32_tiny_tiles = true;
+      else if (fm == 2 && fn == 2) fn = 1;
       const long long tiles = (long long)(a.m / (64 * fm)) * ((a.n + 64 * fn - 1) / (64 * fn)) * a.batch;
       const long long by_k = a.batch == 1 ? std::max(1, (a.k / bk) / 2) : 1;
       if (tiles * by_k * 4 < ctx->num_cus) return kUnsupported;
     }
   }
 
+  // 16-bit types: a workgroup's time is the latency chain of its K loop, not
+  // the matrix pipe, so with 128-wide tiles for at most half of the CUs the
+  // 64 x 64 shape (four times the workgroups, a quarter of the bytes per K
+  // tile each) is faster (1024^3: 9.8 -> 5.4 us; 512^3: 6.7 -> 3.8 us); with
+  // more tiles than that the larger shapes win (1536^3: 13.4 against 16.2 us).
+  if (!f32 && a.m % 64 == 0 && a.n % 64 == 0) {
+    const long long tiles_now = (long long)(a.m / (64 * fm)) * (a.n / (64 * fn)) * a.batch;
+    if (tiles_now * 2 <= ctx->num_cus) fm = 1, fn = 1;
+  }
   MidParams p;
   p.A = a.A;
   p.B = a.B;
@@ -87,7 +107,7 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (f32_small) {
     // fp32 with few tiles: a K tile costs 0.85 us of matrix-pipe time per
     // 128 x 64 tile, so splits down to 2 K tiles still pay for the fold.
-    if (a.batch == 1 && kt_total >= 4) {
+    if (a.batch == 1 && kt_total >= 4 && !f32_tiny_tiles) {
       const size_t per = (size_t)a.m * a.n * sizeof(float);
       long long s = ctx->num_cus / tiles;
       if (s > kt_total / 2) s = kt_total / 2;
@@ -111,6 +131,7 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
   auto launch = [&](int batch, int nsplit, int epi) {
     if (fm == 2 && fn == 2) return launch_shape<2, 2>(ctx, p, a.dtype, batch, nsplit, epi, akc, bkc);
     if (fm == 2) return launch_shape<2, 1>(ctx, p, a.dtype, batch, nsplit, epi, akc, bkc);
+    if (fn == 1) return launch_shape<1, 1>(ctx, p, a.dtype, batch, nsplit, epi, akc, bkc);
     return launch_shape<1, 2>(ctx, p, a.dtype, batch, nsplit, epi, akc, bkc);
   };
   if (splits == 1) return launch(a.batch, 1, general ? kGeneral : kPlain);

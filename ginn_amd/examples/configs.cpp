@@ -505,6 +505,36 @@ long scenario_timed_fills() { return g_timed_fills; }
 // (internal::LateOuterSum in ginn/node/prod.h).
 long scenario_late_sum_columns() { return static_cast<long>(internal::late_outer_sum_columns().load()); }
 
+// `steps` calls of one strided batched product, back to back on the context's
+// stream and issued from native code, after `warmup` untimed ones: a product of
+// a few microseconds can only be timed when the calls arrive faster than they
+// run, which an interpreter's call overhead does not allow.  *out_ms = time per
+// call between two events on that stream.
+int scenario_time_batched_gemm(ginn_hip_ctx* ctx, int dtype, int op_a, int op_b, int m, int n, int k, const void* A,
+                               int lda, long long stride_a, const void* B, int ldb, long long stride_b, float beta,
+                               void* C, int ldc, long long stride_c, int batch, int warmup, int steps,
+                               float* out_ms) {
+  auto call = [&]() {
+    return ginn_hip_gemm_strided_batched(ctx, static_cast<ginn_hip_dtype>(dtype), static_cast<ginn_hip_op>(op_a),
+                                         static_cast<ginn_hip_op>(op_b), m, n, k, A, lda, stride_a, B, ldb, stride_b,
+                                         beta, C, ldc, stride_c, batch);
+  };
+  int rc = 0;
+  for (int i = 0; i < warmup && !rc; ++i) rc = call();
+  if (!rc) rc = ginn_hip_event_record(ctx, 0);
+  for (int i = 0; i < steps && !rc; ++i) rc = call();
+  if (!rc) rc = ginn_hip_event_record(ctx, 1);
+  if (!rc) rc = ginn_hip_sync(ctx);
+  float ms = 0.f;
+  if (!rc) rc = ginn_hip_event_elapsed_ms(ctx, 0, 1, &ms);
+  if (rc) {
+    g_error = ginn_hip_last_error();
+    return rc;
+  }
+  *out_ms = ms / static_cast<float>(steps > 0 ? steps : 1);
+  return 0;
+}
+
 int scenario_mlp(int dtype, int batch, int n_layers, const int* dims, const int* acts, const float* x,
                  const int* labels, const float* const* W, const float* const* b, int iters, float* out_loss,
                  float* out_nll, float* const* dW, float* const* db, float* out_ms) {

@@ -131,10 +131,12 @@ def test_strided_batch(dev, dt, op_a, op_b, beta):
                                    (384, 64, 192), (64, 384, 320), (128, 64, 4096), (4096, 64, 4096),
                                    (64, 4096, 512), (128, 192, 64), (64, 128, 64),
                                    (4096, 16, 4096), (256, 100, 192), (128, 130, 64), (384, 37, 1024),
-                                   (64, 200, 128), (1024, 1000, 256)])
+                                   (64, 200, 128), (1024, 1000, 256), (512, 512, 512), (192, 320, 256),
+                                   (1024, 512, 128), (1024, 1024, 1024)])
 @pytest.mark.parametrize("beta", [0.0, 1.0])
 def test_mid_kernel_shapes(dev, dt, op_a, op_b, m, n, k, beta):
-    """Shapes of the 128 x 128 kernel and its 128 x 64 / 64 x 128 variants: one
+    """Shapes of the 128 x 128 kernel and its 128 x 64 / 64 x 128 / 64 x 64 variants (the last for
+    outputs of few tiles: 512^3, 1024^3, 192 x 320, and with split K 128 x 64 x 4096): one
     tile, odd tile counts (no XCD grouping), one to many K tiles, and long-K /
     few-tile shapes that split K (the weight-gradient products of the GPT layer
     among them), and n that does not fill the last tile column (masked when B
