@@ -280,10 +280,12 @@ int launch_gemm_ksplit(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (a.dtype != GINN_HIP_F32 || a.batch != 1) return kUnsupported;
   if (a.pre && a.ccols) return kUnsupported;
   // Every wave reads its share of both operand panels itself: that pays while a
-  // wave's share of K is what it asks for at once (kDepth steps) and there is
-  // one workgroup per CU at most.  Longer sums and larger outputs belong to the
-  // kernels that share operands through LDS.
-  if (a.k < 32 || a.k > kWaves * kStep * kDepth) return kUnsupported;
+  // wave's share of K is at most twice what it asks for at once (kDepth steps)
+  // and there is one workgroup per CU at most (measured against the kernels
+  // that share operands through LDS and fold a split K in a second launch:
+  // 1024 x 64 x 2048 7.8-9.5 against 12.9 us, 2048 x 128 x 2048 16.2-17.5
+  // against 18.5-19.5 us; 4096 x 64 x 4096 30.9-33.7 against 26.5-27.4 us).
+  if (a.k < 32 || a.k > 2 * kWaves * kStep * kDepth) return kUnsupported;
   const long long tiles = static_cast<long long>((a.m + 31) / 32) * ((a.n + 31) / 32);
   if (tiles > ctx->num_cus) return kUnsupported;
   // A narrow right-hand side under a left operand of several MiB is one pass over that operand at

@@ -74,9 +74,9 @@ def test_reference_prod_golden(dev, golden, dt, op_a, op_b):
 @pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 5, 7), (64, 64, 64), (65, 63, 33), (128, 128, 128),
                                    (200, 136, 72), (129, 257, 100), (10, 64, 512), (512, 64, 784),
                                    # fp32: one launch with K split inside the workgroup, up to its limits
-                                   # (256 tiles of 32 x 32, K = 1024) and just beyond
+                                   # (256 tiles of 32 x 32, K = 2048) and just beyond
                                    (33, 31, 36), (1024, 256, 384), (384, 250, 1024), (500, 500, 1000),
-                                   (96, 40, 1028),
+                                   (96, 40, 1028), (256, 64, 2048), (130, 100, 1900), (128, 64, 2052),
                                    # ... on 16 x 16 tiles (few large tiles, a long sum), ragged edges
                                    (384, 120, 1024), (50, 19, 520), (17, 250, 1000)])
 @pytest.mark.parametrize("beta", [0.0, 1.0])
