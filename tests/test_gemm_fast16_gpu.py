@@ -125,6 +125,30 @@ def test_strided_batch(dev, dt, op_a, op_b, beta):
 
 
 @pytest.mark.parametrize("dt", [capi.F16, capi.BF16, capi.F32])
+@pytest.mark.parametrize("op_a,op_b", [(0, 0), (0, 1), (1, 0)])
+@pytest.mark.parametrize("m,n,k,batch", [(256, 256, 192, 6), (128, 384, 320, 3), (512, 512, 128, 2)])
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_strided_batch_of_few_tiles(dev, dt, op_a, op_b, m, n, k, batch, beta):
+    """Batches whose slices together have few 128-wide tiles: the 64 x 64 tile shape of the mid-size
+    kernel with a batch index (fp32: 96 .. 128 tiles of 64 x 64 without a K split)."""
+    from gpu_util import torch_dtype
+    torch = dev.torch
+    A, B, lda, ldb = _operands(dev, dt, op_a, op_b, m, n, k, batch, 5 + batch)
+    g = torch.Generator(device="cuda").manual_seed(k)
+    C = torch.randn(batch, n, m, generator=g, device="cuda").to(torch_dtype(dt))
+    want = _expected(A, B, op_a, op_b)
+    if beta:
+        want = want + C.double().transpose(1, 2)
+    dev.lib.call("ginn_hip_gemm_strided_batched", dev.ctx, dt, op_a, op_b, m, n, k,
+                 ctypes.c_void_p(A.data_ptr()), lda, A.shape[1] * A.shape[2],
+                 ctypes.c_void_p(B.data_ptr()), ldb, B.shape[1] * B.shape[2], beta,
+                 ctypes.c_void_p(C.data_ptr()), m, m * n, batch)
+    dev.sync()
+    got = C.double().transpose(1, 2)
+    assert float((got - want).norm() / want.norm()) <= _bound(dt)
+
+
+@pytest.mark.parametrize("dt", [capi.F16, capi.BF16, capi.F32])
 @pytest.mark.parametrize("op_a,op_b", [(0, 0), (0, 1), (1, 0), (1, 1)])
 @pytest.mark.parametrize("m,n,k", [(128, 128, 64), (384, 640, 192), (1024, 1024, 512), (2048, 2048, 128),
                                    (768, 768, 4096), (256, 128, 1024), (768, 4096, 768), (128, 256, 8192),
