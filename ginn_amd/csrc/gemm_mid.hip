@@ -72,7 +72,10 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
   // 128 x 64 tiles.
   if (!f32 && a.m % 64 == 0 && (a.n % 64 == 0 || (any_n && a.n > 8))) {
     const long long tiles_now = (long long)(a.m / (64 * fm)) * ((a.n + 64 * fn - 1) / (64 * fn)) * a.batch;
-    if (tiles_now * 2 <= ctx->num_cus) fm = 1, fn = 1;
+    const long long tiles64 = (long long)(a.m / 64) * ((a.n + 63) / 64) * a.batch;
+    // (Two 64 x 64 workgroups per CU over a very long K run level with one 128-wide one:
+    // 2048 x 1024 x 8192 49-57 against 51-52 us; those keep the larger shape.)
+    if (tiles_now * 2 <= ctx->num_cus && !(tiles64 > ctx->num_cus && a.k / bk > 64)) fm = 1, fn = 1;
   }
   MidParams p;
   p.A = a.A;
