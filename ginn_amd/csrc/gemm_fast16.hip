@@ -16,8 +16,12 @@
 //     position = chunk ^ ((row >> 1) & 7); a lane's MFMA operand (8 k of one
 //     row) is one ds_read_b128.
 //   row-contiguous operand ("RC": A, or B^T): [64 k][32 chunks]; chunk
-//     position = chunk ^ (2 * (k & 3)); a lane's operand is two
-//     ds_read_b64_tr_b16 (the 16-lane transposing read of gfx950).
+//     position = chunk ^ (4 * (k & 3)); a lane's operand is two
+//     ds_read_b64_tr_b16 (the 16-lane transposing read of gfx950).  A
+//     transposing read serves 32 lanes per cycle = two 16-lane groups x 4
+//     k-rows x 32 bytes; the k-rows lie 512 bytes apart (the same banks), and
+//     the XOR moves row i by 64 i bytes, so the four rows' 64 bytes fall into
+//     four different quarters of the 64 banks.
 #include <cstdlib>
 #include <type_traits>
 #include <utility>
@@ -62,7 +66,7 @@ struct FastParams {
 };
 
 __device__ __forceinline__ int swz_kc(int row) { return (row >> 1) & 7; }
-__device__ __forceinline__ int swz_rc(int kr) { return 2 * (kr & 3); }
+__device__ __forceinline__ int swz_rc(int kr) { return 4 * (kr & 3); }
 
 // Element offset, relative to the tile origin at K offset 0, of the 16-byte
 // chunk that lands at linear LDS chunk position v of the tile.
