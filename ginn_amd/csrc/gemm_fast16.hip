@@ -536,9 +536,11 @@ int launch_gemm_fast16(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (a.bias && reinterpret_cast<uintptr_t>(a.bias) % 8) return kUnsupported;
   if (a.batch > 1 && (a.stride_a % 8 || a.stride_b % 8 || a.stride_c % 8)) return kUnsupported;
   const long long tiles = (long long)(a.m / BM) * (a.n / BN);
-  // Fewer tiles than three quarters of the CUs leave too much of the chip
-  // idle: the 128 x 128 kernel is the better fit there.
-  if (tiles * a.batch < (ctx->num_cus * 3) / 4) return kUnsupported;
+  // With tiles for fewer than 9/16 of the CUs too much of the chip idles and
+  // the 128 x 128 kernel is the better fit (measured, bf16: 3072^3 = 144 tiles
+  // 61 us here against 78-79 us there; 2048 x 4096 x 2048 = 128 tiles level at
+  // 42-43 us; 2560^3 = 100 tiles 51-55 against 46 us).
+  if (tiles * a.batch * 16 < ctx->num_cus * 9) return kUnsupported;
   // Per-lane byte offsets inside one operand tile are kept in 32 bits.
   if ((long long)a.lda * 256 * 2 >= (1ll << 31) || (long long)a.ldb * 256 * 2 >= (1ll << 31))
     return kUnsupported;

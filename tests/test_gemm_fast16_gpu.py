@@ -77,6 +77,27 @@ def test_pipeline_lengths(dev, dt, op_a, op_b, k, beta):
 
 @pytest.mark.parametrize("dt", [capi.F16, capi.BF16])
 @pytest.mark.parametrize("op_a,op_b", [(0, 0), (0, 1), (1, 0)])
+@pytest.mark.parametrize("m,n,k", [(3072, 3072, 320), (2304, 4096, 256), (3328, 2816, 384)])
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_fewest_tiles_of_the_large_kernel(dev, dt, op_a, op_b, m, n, k, beta):
+    """144 tiles of 256 x 256 (the fewest the 256 x 256 kernel takes: 12 x 12 and 9 x 16) and 143
+    (13 x 11, one short: the 128 x 128 kernel)."""
+    from gpu_util import TIGHT, torch_dtype
+    torch = dev.torch
+    A, B, lda, ldb = _operands(dev, dt, op_a, op_b, m, n, k, 1, m + n)
+    g = torch.Generator(device="cuda").manual_seed(n)
+    C = torch.randn(1, n, m, generator=g, device="cuda").to(torch_dtype(dt))
+    want = _expected(A, B, op_a, op_b)
+    if beta:
+        want = want + beta * C.double().transpose(1, 2)
+    dev.gemm(dt, op_a, op_b, m, n, k, A.data_ptr(), lda, B.data_ptr(), ldb, beta, C.data_ptr(), m)
+    dev.sync()
+    err = float((C.double().transpose(1, 2) - want).norm() / want.norm())
+    assert err <= TIGHT[dt], err
+
+
+@pytest.mark.parametrize("dt", [capi.F16, capi.BF16])
+@pytest.mark.parametrize("op_a,op_b", [(0, 0), (0, 1), (1, 0)])
 def test_rectangular_and_padded_ld(dev, dt, op_a, op_b):
     """m != n, leading dimensions larger than the row counts."""
     from gpu_util import TIGHT, torch_dtype
