@@ -118,16 +118,22 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_kernel(int rows, int col
 // dgamma += sum_c dz (*) y and dbeta += sum_c dz stay in registers over the
 // columns of a wave and leave as one fp32 partial row per workgroup.  One wave
 // per column, rows <= 64 * V * ITERS (ITERS vectors per lane; at most kLnRowIters).
+// A column is one load -> two wave sums -> store chain, and the waves on a CU
+// are all the chains it overlaps: workgroups of 8 waves (up to 256 registers
+// each: the longest columns keep 5 x 32 values per lane), at most two per CU,
+// a partial row each (768 x 4096 bf16: 17.3 us with one workgroup of 4 waves
+// per CU, four columns one after the other in each wave).
 constexpr int kLnRowIters = 4;
+constexpr int kLnBwdWaves = 8;
 template <typename T, int V, int ITERS>
-__global__ __launch_bounds__(kBlock) void layernorm_affine_bwd_kernel(
+__global__ __launch_bounds__(kLnBwdWaves * 64) void layernorm_affine_bwd_kernel(
     int rows, int cols, const typename T::storage* __restrict__ dz, const typename T::storage* __restrict__ y,
     const float* __restrict__ std_in, const typename T::storage* __restrict__ gamma, float mb,
     typename T::storage* dx, int accumulate, float* __restrict__ part_g, float* __restrict__ part_b) {
-  __shared__ float red[kWaves][64 * V];
+  __shared__ float red[kLnBwdWaves][64 * V];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int wave = blockIdx.x * kWaves + w;
-  const int nwaves = gridDim.x * kWaves;
+  const int wave = blockIdx.x * kLnBwdWaves + w;
+  const int nwaves = gridDim.x * kLnBwdWaves;
   const float inv_rows = 1.f / static_cast<float>(rows);
   float scale[ITERS][V], sg[ITERS][V], sb[ITERS][V];
 #pragma unroll
@@ -183,7 +189,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_affine_bwd_kernel(
     }
   }
   if (!part_g) return;
-  // The four waves' row sums -> one partial row per workgroup (waves 1..3 hand theirs to wave 0).
+  // The waves' row sums -> one partial row per workgroup (the others hand theirs to wave 0).
 #pragma unroll
   for (int which = 0; which < 2; ++which) {
 #pragma unroll
@@ -200,7 +206,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_affine_bwd_kernel(
         for (int e = 0; e < V; ++e) {
           float t = 0.f;
 #pragma unroll
-          for (int k = 0; k < kWaves; ++k) t += red[k][lane * V + e];
+          for (int k = 0; k < kLnBwdWaves; ++k) t += red[k][lane * V + e];
           out[e] = t;
         }
       }
@@ -573,9 +579,9 @@ int ginn_hip_layernorm_affine_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int r
     return rc != kOk ? rc : rc_free;
   }
   std::lock_guard<std::mutex> lock(ctx->mutex);
-  // At most one workgroup per CU: every workgroup leaves a partial row for the fold.
-  unsigned grid = grid_for(static_cast<size_t>(cols), kWaves, ctx->num_cus);
-  const unsigned cap = static_cast<unsigned>(ctx->num_cus);
+  // At most two workgroups per CU: every workgroup leaves a partial row for the fold.
+  unsigned grid = grid_for(static_cast<size_t>(cols), kLnBwdWaves, ctx->num_cus);
+  const unsigned cap = 2 * static_cast<unsigned>(ctx->num_cus);
   if (grid > cap) grid = cap;
   const size_t part_bytes = static_cast<size_t>(grid) * rows * sizeof(float);
   rowred::Partials room{nullptr, false};
@@ -588,7 +594,7 @@ int ginn_hip_layernorm_affine_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int r
   float* part_b = part_g ? part_g + static_cast<size_t>(grid) * rows : nullptr;
   const int iters = (rows + per_iter - 1) / per_iter;
 #define GH_LN_BWD(ITERS)                                                                                       \
-  GH_DISPATCH_DTYPE_V(dtype, vec, (layernorm_affine_bwd_kernel<T, V, ITERS><<<grid, kBlock, 0, ctx->stream>>>( \
+  GH_DISPATCH_DTYPE_V(dtype, vec, (layernorm_affine_bwd_kernel<T, V, ITERS><<<grid, kLnBwdWaves * 64, 0, ctx->stream>>>( \
       rows, cols, static_cast<const T::storage*>(dz), static_cast<const T::storage*>(y), std_in,              \
       static_cast<const T::storage*>(gamma), multiplier_bias, static_cast<T::storage*>(dx), accumulate,       \
       part_g, part_b)))
