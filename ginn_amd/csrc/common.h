@@ -9,6 +9,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <map>
+#include <atomic>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -145,6 +146,17 @@ struct BF16 {
   using storage = uint16_t;
   static constexpr int kDtype = GINN_HIP_BF16;
 };
+
+// Raises a kernel's limit of dynamic LDS once per device and kernel (`done`
+// is that kernel's own mask of devices): the runtime call costs the host most
+// of a microsecond, which a product of a few microseconds cannot hide.
+inline hipError_t allow_dynamic_lds(std::atomic<unsigned long long>& done, int device, const void* fn, int bytes) {
+  const unsigned long long bit = 1ull << (device & 63);
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
 
 inline size_t dtype_size(int dtype) { return dtype == GINN_HIP_F32 ? 4 : 2; }
 inline bool dtype_valid(int dtype) {

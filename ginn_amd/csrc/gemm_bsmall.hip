@@ -244,8 +244,8 @@ int launch_one(ginn_hip_ctx* ctx, const Params& p) {
   const int stages = p.k / 64 > 1 ? 2 : 1;
   const int lds_bytes = G::lds_bytes(stages);
   auto fn = gemm_bsmall_kernel<T, AKC, BKC, FM, FN>;
-  GH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                             G::lds_bytes(2)));
+  static std::atomic<unsigned long long> lds_allowed{0};
+  GH_HIP(allow_dynamic_lds(lds_allowed, ctx->device, reinterpret_cast<const void*>(fn), G::lds_bytes(2)));
   const long long blocks = (long long)p.tiles_m * p.tiles_n * p.batch;
   fn<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreadsB), lds_bytes, ctx->stream>>>(p);
   GH_HIP(hipGetLastError());

@@ -500,13 +500,13 @@ int launch_epi(ginn_hip_ctx* ctx, const FastParams& p, int batch, bool general) 
   const dim3 grid(p.tiles_m * p.tiles_n, batch);
   if (general) {
     auto fn = gemm_fast16_kernel<T, AKC, BKC, true>;
-    GH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
+    static std::atomic<unsigned long long> lds_allowed{0};
+    GH_HIP(allow_dynamic_lds(lds_allowed, ctx->device, reinterpret_cast<const void*>(fn), kLdsBytes));
     fn<<<grid, dim3(kThreads), kLdsBytes, ctx->stream>>>(p);
   } else {
     auto fn = gemm_fast16_kernel<T, AKC, BKC, false>;
-    GH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
+    static std::atomic<unsigned long long> lds_allowed{0};
+    GH_HIP(allow_dynamic_lds(lds_allowed, ctx->device, reinterpret_cast<const void*>(fn), kLdsBytes));
     fn<<<grid, dim3(kThreads), kLdsBytes, ctx->stream>>>(p);
   }
   GH_HIP(hipGetLastError());

@@ -669,8 +669,9 @@ int launch_epi(ginn_hip_ctx* ctx, const MidParams& p, int batch, int splits, int
 #define GH_MID_LAUNCH(E)                                                                          \
   {                                                                                               \
     auto fn = gemm_mid_kernel<T, AKC, BKC, E, FM, FN>;                                          \
-    GH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(fn),                                 \
-                               hipFuncAttributeMaxDynamicSharedMemorySize, G::kLdsBytes));        \
+    static std::atomic<unsigned long long> lds_allowed{0};                                        \
+    GH_HIP(allow_dynamic_lds(lds_allowed, ctx->device, reinterpret_cast<const void*>(fn),         \
+                             G::kLdsBytes));                                                      \
     fn<<<grid, dim3(kThreads), lds_bytes, ctx->stream>>>(p);                                      \
   }
   if (epi == kPartial) GH_MID_LAUNCH(kPartial)
