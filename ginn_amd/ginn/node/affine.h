@@ -8,6 +8,8 @@
 #ifndef GINN_NODE_AFFINE_H
 #define GINN_NODE_AFFINE_H
 
+#include <optional>
+
 #include <ginn/node/data.h>
 #include <ginn/nonlin.h>
 #include <ginn/prod.h>
@@ -59,6 +61,8 @@ class AffineNode : public BaseDataNode<Scalar> {
                                       value().data()));
   }
 
+  static constexpr double kBesideRowSum = 1048576.;  // elements from which a row sum is worth a second stream
+
   void backward_() override {
     using namespace internal;
     const bool identity = nonlin_->is_identity();
@@ -66,8 +70,16 @@ class AffineNode : public BaseDataNode<Scalar> {
     if (!identity) dpreactiv_.resize(grad().shape());
     auto& bias = ins_.back();
     const Size m = grad().rows(), n = grad().cols();
-    PostponeFolds later(ctx_of(grad()), *bias);  // the bias gradient is complete when the pass ends
-    GINN_HIP_CALL(ginn_hip_affine_bwd_pre(ctx_of(grad()), dtype_of<Scalar>(), nonlin_->code(),
+    // Without an activation this call is the row sum for the bias gradient alone and nothing in the
+    // pass waits for it: a large one runs beside the pass like the weight gradients below (and folds
+    // at once there: the folds that wait for the end of the pass are flushed on the pass's own stream).
+    ginn_hip_ctx* pre_ctx = ctx_of(grad());
+    if (identity && bias->has_grad() && static_cast<double>(m) * static_cast<double>(n) >= kBesideRowSum)
+      pre_ctx = BesidePass::ctx_for(*bias, dev(), BesidePass::kWorthIt);
+    const bool beside = pre_ctx != ctx_of(grad());
+    std::optional<PostponeFolds> later;  // the bias gradient is complete when the pass ends
+    if (!beside) later.emplace(pre_ctx, *bias);
+    GINN_HIP_CALL(ginn_hip_affine_bwd_pre(pre_ctx, dtype_of<Scalar>(), nonlin_->code(),
                                           static_cast<int>(m), static_cast<int>(n), grad().data(),
                                           value().data(), preactiv_.size() > 0 ? preactiv_.data() : nullptr,
                                           identity ? nullptr : dpreactiv_.data(),

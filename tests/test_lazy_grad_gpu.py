@@ -124,9 +124,10 @@ def test_only_single_overwriting_users_qualify(shim):
 def test_weight_gradients_beside_the_pass_are_the_same_bits(shim, dt, mode):
     """Products of >= 1 GFLOP into the gradients of weights run on the GPU's second stream while a
     backward pass runs (internal::BesidePass in ginn_amd/ginn/node.h; the reference has one stream,
-    ginn/dev.h:188-189).  Same kernels on the same operands: after three passes without a wait in
-    between, loss and every gradient are bit-identical to the run on one stream."""
-    sizes = dict(hs=64, nh=12, B=4, T=256, V=1024)  # 768 x 768 x 1024 products: 1.2 GFLOP each
+    ginn/dev.h:188-189), and so do the bias row sums of Affines without an activation from 2^20
+    elements on (ginn_amd/ginn/node/affine.h).  Same kernels on the same operands: after three passes
+    without a wait in between, loss and every gradient are bit-identical to the run on one stream."""
+    sizes = dict(hs=64, nh=12, B=4, T=512, V=1024)  # 768 x 768 x 2048 products: 2.4 GFLOP; 768 x 2048 row sums
     try:
         shim.shim_set_beside_pass(0)
         want_loss, want_dx, want_grads, _, _ = run(shim, dt, 1, mode, 3, seed=11, **sizes)
