@@ -1,6 +1,6 @@
 """Parity of the tuned kernels against an fp64 product of the same rounded
 inputs (fp16 / bf16: both kernels; fp32: the mid-size kernel).  The 256 x 256 x 64 kernel is taken for m, n multiples of
-256, k a multiple of 64 and at least 256, and at least 192 tiles; the
+256, k a multiple of 64 and at least 256, and at least 144 tiles; the
 128 x 128 x 64 kernel (optionally split-K) for the remaining shapes with m, n
 multiples of 128 and k of 64.  Covered: every pipeline length with its own code
 path, all four layouts, plain and accumulating epilogues, padded leading
@@ -291,3 +291,43 @@ def test_mid_kernel_attention_batches(dev, dt, op_a, op_b, m, n, k):
     dev.sync()
     got = C.double().transpose(1, 2)
     assert float((got - want).norm() / want.norm()) <= _bound(dt)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+def test_seeded_random_shapes(dev, seed):
+    """Which kernel takes a product is decided by its extents, type, layout and batch (tile counts against
+    the number of CUs, K against the split limits): 250 seeded draws per case from extents on both sides of
+    every such limit, aligned and ragged, all four layouts, beta 0 / 0.5 / 1, some as strided batches, each
+    against the fp64 product of the same rounded operands."""
+    import random
+    from gpu_util import torch_dtype
+    torch = dev.torch
+    rng = random.Random(seed)
+    ms = [64, 128, 192, 256, 320, 384, 512, 640, 768, 1024, 1280, 1536, 2048, 2304, 3072, 4096, 100, 200, 1000, 33]
+    ns = ms + [1, 4, 8, 9, 16, 37, 40, 72, 130]
+    ks = [32, 64, 96, 128, 192, 256, 320, 512, 768, 1024, 1056, 1536, 2048, 2052, 3072, 4096, 100, 1000]
+    worst = {}
+    for it in range(250):
+        dt = rng.choice([capi.F32, capi.F16, capi.BF16])
+        m, n, k = rng.choice(ms), rng.choice(ns), rng.choice(ks)
+        op_a, op_b = rng.choice([(0, 0), (0, 1), (1, 0), (1, 1)])
+        beta = rng.choice([0.0, 1.0, 0.5])
+        if m * n * k > 3e10 or m * n > 2 ** 24:
+            continue
+        batch = rng.choice([1, 1, 1, 2, 5]) if m * n * k < 2e9 else 1
+        A, B, lda, ldb = _operands(dev, dt, op_a, op_b, m, n, k, batch, 1000 * seed + it)
+        g = torch.Generator(device="cuda").manual_seed(it)
+        C = torch.randn(batch, n, m, generator=g, device="cuda").to(torch_dtype(dt))
+        want = _expected(A, B, op_a, op_b) + beta * C.double().transpose(1, 2)
+        if batch == 1:
+            dev.gemm(dt, op_a, op_b, m, n, k, A.data_ptr(), lda, B.data_ptr(), ldb, beta, C.data_ptr(), m)
+        else:
+            dev.lib.call("ginn_hip_gemm_strided_batched", dev.ctx, dt, op_a, op_b, m, n, k,
+                         ctypes.c_void_p(A.data_ptr()), lda, A.shape[1] * A.shape[2],
+                         ctypes.c_void_p(B.data_ptr()), ldb, B.shape[1] * B.shape[2], beta,
+                         ctypes.c_void_p(C.data_ptr()), m, m * n, batch)
+        dev.sync()
+        err = float((C.double().transpose(1, 2) - want).norm() / want.norm())
+        assert err <= 2 * _bound(dt), (dt, op_a, op_b, m, n, k, batch, beta, err)
+        worst[dt] = max(worst.get(dt, 0.0), err)
+    assert len(worst) == 3
