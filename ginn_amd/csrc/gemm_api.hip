@@ -36,6 +36,90 @@ int check_gemm_args(const char* who, const GemmArgs& a) {
   return kOk;
 }
 
+// Extents that are no multiples of the tuned kernels' tiles (4000^3; m = 1000) left a product on
+// the any-shape kernel, several times slower than its aligned neighbours (fp16 4000^3: 596 us
+// against 112 us for 4096^3).  With leading dimensions and pointers that allow 16-byte accesses the
+// product is cut instead: the last K % (K tile) values over the whole output first (any-shape
+// kernel, the caller's beta), then the aligned core (tuned kernels) and the ragged rows and columns
+// around it (any-shape kernel) over the whole K tiles, adding to that, with the caller's epilogue.
+// A 16-bit sum is then rounded to the storage type once in between, as between the (W, X) pairs of
+// an Affine.
+int launch_gemm_ragged(ginn_hip_ctx* ctx, const GemmArgs& a) {
+  if (a.batch != 1 || a.acols || a.bcols || a.ccols) return kUnsupported;
+  const long long es = static_cast<long long>(dtype_size(a.dtype));
+  const int per16 = static_cast<int>(16 / es), bk = static_cast<int>(128 / es);
+  if (a.lda % per16 || a.ldb % per16 || a.ldc % per16) return kUnsupported;
+  auto aligned16 = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
+  if (!aligned16(a.A) || !aligned16(a.B) || !aligned16(a.C) || (a.pre && !aligned16(a.pre)) ||
+      (a.bias && !aligned16(a.bias)))
+    return kUnsupported;
+  const int m0 = a.m / 128 * 128, k0 = a.k / bk * bk;
+  // With a K-contiguous B the tuned kernels mask a partly filled last tile column themselves.
+  const int n0 = a.op_b == GINN_HIP_OP_N ? a.n : a.n / 128 * 128;
+  if (m0 == a.m && n0 == a.n && k0 == a.k) return kUnsupported;
+  if (m0 < 256 || n0 < 256 || k0 < 4 * bk) return kUnsupported;
+  // Worth the extra launches: a core of at least 512^3 multiply-adds that is most of the product.  Ragged
+  // rows cost more than a ragged K (their few rows times all of K are a slow shape for the any-shape
+  // kernel): only from 4 (fp32) or 8 x as much on, and not for the 16-bit types with a K-contiguous A, where
+  // the any-shape kernel alone is as fast (measured, us before -> after: fp16 NN 4000^3 596 -> 365,
+  // 2000^3 106 -> 59, 1024 x 1024 x 1000 20.6 -> 11.7; fp32 NN 4000^3 1220 -> 1097, 2000^3 242 -> 185,
+  // 1000 x 1024 x 1024 42.7 -> 29.8; but fp16 TN 4000^3 239 -> 357, 1000^3 14.6 -> 21.2).
+  const double core = static_cast<double>(m0) * n0 * k0, all = static_cast<double>(a.m) * a.n * a.k;
+  if (core < 134217728. || core < 0.75 * all) return kUnsupported;
+  const bool f32 = a.dtype == GINN_HIP_F32;
+  if (m0 < a.m && (core < (f32 ? 536870912. : 1073741824.) || (!f32 && a.op_a == GINN_HIP_OP_T))) return kUnsupported;
+
+  const char* A = static_cast<const char*>(a.A);
+  const char* B = static_cast<const char*>(a.B);
+  const bool at = a.op_a == GINN_HIP_OP_T, bt = a.op_b == GINN_HIP_OP_T;
+  // Byte offsets of row r / K index kk of op(A), column c / K index kk of op(B), element (r, c) of C.
+  auto a_at = [&](long long r, long long kk) { return A + (at ? r * a.lda + kk : kk * a.lda + r) * es; };
+  auto b_at = [&](long long kk, long long c) { return B + (bt ? kk * a.ldb + c : c * a.ldb + kk) * es; };
+  auto c_at = [&](void* base, long long r, long long c) {
+    return base ? static_cast<void*>(static_cast<char*>(base) + (c * a.ldc + r) * es) : nullptr;
+  };
+  float beta = a.beta;
+  if (k0 < a.k) {
+    GemmArgs t = a;
+    t.k = a.k - k0;
+    t.A = a_at(0, k0);
+    t.B = b_at(k0, 0);
+    t.bias = nullptr;
+    t.act = GINN_HIP_ACT_IDENTITY;
+    if (int rc = launch_gemm_generic(ctx, t)) return rc;
+    beta = 1.f;
+  }
+  GemmArgs c = a;
+  c.m = m0;
+  c.n = n0;
+  c.k = k0;
+  c.beta = beta;
+  if (int rc = launch_gemm(ctx, c)) return rc;
+  if (n0 < a.n) {  // the columns right of the core, all rows
+    GemmArgs f = a;
+    f.n = a.n - n0;
+    f.k = k0;
+    f.beta = beta;
+    f.B = b_at(0, n0);
+    f.C = c_at(a.C, 0, n0);
+    f.pre = c_at(a.pre, 0, n0);
+    if (int rc = launch_gemm(ctx, f)) return rc;
+  }
+  if (m0 < a.m) {  // the rows below the core, its columns
+    GemmArgs f = a;
+    f.m = a.m - m0;
+    f.n = n0;
+    f.k = k0;
+    f.beta = beta;
+    f.A = a_at(m0, 0);
+    f.C = c_at(a.C, m0, 0);
+    f.pre = c_at(a.pre, m0, 0);
+    if (a.bias) f.bias = static_cast<const char*>(a.bias) + static_cast<long long>(m0) * es;
+    if (int rc = launch_gemm(ctx, f)) return rc;
+  }
+  return kOk;
+}
+
 }  // namespace
 
 int launch_gemm(ginn_hip_ctx* ctx, const GemmArgs& a) {
@@ -68,6 +152,8 @@ int launch_gemm(ginn_hip_ctx* ctx, const GemmArgs& a) {
   rc = launch_gemm_bsmall(ctx, a);
   if (rc != kUnsupported) return rc;
   rc = launch_gemm_mid(ctx, a);
+  if (rc != kUnsupported) return rc;
+  rc = launch_gemm_ragged(ctx, a);
   if (rc != kUnsupported) return rc;
   return launch_gemm_generic(ctx, a);
 }

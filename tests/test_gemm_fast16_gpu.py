@@ -331,3 +331,24 @@ def test_seeded_random_shapes(dev, seed):
         assert err <= 2 * _bound(dt), (dt, op_a, op_b, m, n, k, batch, beta, err)
         worst[dt] = max(worst.get(dt, 0.0), err)
     assert len(worst) == 3
+
+
+@pytest.mark.parametrize("dt", [capi.F32, capi.F16, capi.BF16])
+@pytest.mark.parametrize("op_a,op_b", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(1024, 1024, 1000), (2000, 2000, 2000), (1000, 1024, 1024), (1160, 1096, 1032),
+                                   (1024, 520, 4100)])
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_ragged_extents_with_aligned_leading_dimensions(dev, dt, op_a, op_b, m, n, k, beta):
+    """Extents that are no multiples of the tuned kernels' tiles while leading dimensions and pointers
+    allow 16-byte accesses: the product is cut into the last K % 64 (32 for fp32) values over the whole
+    output, the aligned core on the tuned kernels, and the ragged rows / columns around it."""
+    from gpu_util import torch_dtype
+    torch = dev.torch
+    A, B, lda, ldb = _operands(dev, dt, op_a, op_b, m, n, k, 1, m + n + k)
+    g = torch.Generator(device="cuda").manual_seed(k)
+    C = torch.randn(1, n, m, generator=g, device="cuda").to(torch_dtype(dt))
+    want = _expected(A, B, op_a, op_b) + beta * C.double().transpose(1, 2)
+    dev.gemm(dt, op_a, op_b, m, n, k, A.data_ptr(), lda, B.data_ptr(), ldb, beta, C.data_ptr(), m)
+    dev.sync()
+    err = float((C.double().transpose(1, 2) - want).norm() / want.norm())
+    assert err <= 2 * _bound(dt), err
