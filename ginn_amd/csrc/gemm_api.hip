@@ -54,17 +54,15 @@ int launch_gemm_ragged(ginn_hip_ctx* ctx, const GemmArgs& a) {
       (a.bias && !aligned16(a.bias)))
     return kUnsupported;
   const int m0 = a.m / 128 * 128, k0 = a.k / bk * bk;
-  // With a K-contiguous B the tuned kernels mask a partly filled last tile column themselves; they take
-  // 128 x 64 tiles for the whole product when it is less than half full, which costs more than cutting it off.
-  const bool masked_ok = a.op_b == GINN_HIP_OP_N && (a.n - 1) % 128 >= 64;
-  const int n0 = masked_ok ? a.n : a.n / 128 * 128;
+  // With a K-contiguous B the tuned kernels mask a partly filled last tile column themselves.
+  const int n0 = a.op_b == GINN_HIP_OP_N ? a.n : a.n / 128 * 128;
   if (m0 == a.m && n0 == a.n && k0 == a.k) return kUnsupported;
   if (m0 < 256 || n0 < 256 || k0 < 4 * bk) return kUnsupported;
   // Worth the extra launches: a core of at least 512^3 multiply-adds that is most of the product.  Ragged
   // rows cost more than a ragged K (their few rows times all of K are a slow shape for the any-shape
   // kernel): only from 4 (fp32) or 8 x as much on, and not for the 16-bit types with a K-contiguous A, where
-  // the any-shape kernel alone is as fast (measured, us before -> after: fp16 NN 4000^3 596 -> 259,
-  // 2000^3 106 -> 59, 1024 x 1024 x 1000 20.6 -> 11.7; fp32 NN 4000^3 1220 -> 1097, 2000^3 242 -> 185,
+  // the any-shape kernel alone is as fast (measured, us before -> after: fp16 NN 4000^3 596 -> 217,
+  // 2000^3 106 -> 59, 1024 x 1024 x 1000 20.6 -> 11.7; fp32 NN 4000^3 1220 -> 996, 2000^3 242 -> 185,
   // 1000 x 1024 x 1024 42.7 -> 29.8; but fp16 TN 4000^3 239 -> 357, 1000^3 14.6 -> 21.2).
   const double core = static_cast<double>(m0) * n0 * k0, all = static_cast<double>(a.m) * a.n * a.k;
   if (core < 134217728. || core < 0.75 * all) return kUnsupported;
