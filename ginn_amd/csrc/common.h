@@ -109,6 +109,7 @@ struct ginn_hip_ctx {
   std::mutex mutex;  // serialises workspace users across host threads
   hipEvent_t events[64] = {};
   int num_cus = 256;
+  bool may_allocate = true;  // false for the stack context of the entry point that must not allocate
   ginn_hip_pool pool;
   ginn_hip_fold_queue folds;  // guarded by `mutex`
 };

@@ -36,6 +36,85 @@ int check_gemm_args(const char* who, const GemmArgs& a) {
   return kOk;
 }
 
+// A leading dimension or pointer that rules out 16-byte accesses -- an odd row count as the leading
+// dimension of a column-major operand is enough -- leaves a product on the any-shape kernel's element
+// loads: 20 x slower than its aligned neighbour for a large one (fp16 4095 x 4097 x 4099: 2.6-2.9 ms
+// against 0.11 ms for 4096^3).  A large product is therefore computed on copies with padded leading
+// dimensions (blocks from the context's pool, released after the calls: reuse is ordered on the stream):
+// the operands that need it are copied in, the output (and the kept pre-activation) copied in when beta
+// reads it and copied back afterwards.  Not while the stream is being captured (the pool may have to
+// allocate) and not for the entry point that must not allocate.
+int launch_gemm_realigned(ginn_hip_ctx* ctx, const GemmArgs& a) {
+  if (a.batch != 1 || a.acols || a.bcols || a.ccols || !ctx->may_allocate) return kUnsupported;
+  const size_t es = dtype_size(a.dtype);
+  const int per16 = static_cast<int>(16 / es);
+  auto bad = [&](const void* ptr, int ld) { return reinterpret_cast<uintptr_t>(ptr) % 16 != 0 || ld % per16 != 0; };
+  const bool fix_a = bad(a.A, a.lda), fix_b = bad(a.B, a.ldb);
+  const bool fix_c = bad(a.C, a.ldc) || (a.pre && bad(a.pre, a.ldc));
+  const bool fix_bias = a.bias && reinterpret_cast<uintptr_t>(a.bias) % 16 != 0;
+  if (!fix_a && !fix_b && !fix_c && !fix_bias) return kUnsupported;
+  // From where the copies pay (measured, any-shape kernel alone -> on copies, us): fp32 1001 x 1003 x 1005
+  // 115 -> 56, 515 x 2049 x 515 75 -> 47, but 801 x 803 x 805 54 -> 62; fp16 with one operand to copy
+  // 1024 x 1024 x 1001 73 -> 20, with all three 1501 x 1503 x 1505 181 -> 79 but 1001 x 1003 x 1005 74 -> 91.
+  const int copies = int(fix_a) + int(fix_b) + int(fix_c);
+  const double work = static_cast<double>(a.m) * a.n * a.k;
+  const double least = a.dtype == GINN_HIP_F32 ? 536870912. : (copies >= 2 ? 2147483648. : 268435456.);
+  if (a.m < 256 || a.n < 256 || a.k < 256 || work < least) return kUnsupported;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  GH_HIP(hipStreamIsCapturing(ctx->stream, &capturing));
+  if (capturing != hipStreamCaptureStatusNone) return kUnsupported;
+
+  const ginn_hip_dtype dt = static_cast<ginn_hip_dtype>(a.dtype);
+  void* blocks[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+  int used = 0;
+  auto padded = [](int rows) { return (rows + 63) / 64 * 64; };
+  // A copy of the stored rows x cols matrix at src with a padded leading dimension (filled when `fill`).
+  auto take = [&](const void* src, int rows, int cols, int ld, bool fill, void** out, int* ld_out) {
+    *ld_out = padded(rows);
+    int rc = ginn_hip_malloc(ctx, static_cast<size_t>(*ld_out) * cols * es, out);
+    if (rc != kOk) return rc;
+    blocks[used++] = *out;
+    return fill ? ginn_hip_copy_2d(ctx, dt, rows, cols, src, ld, *out, *ld_out, 0) : kOk;
+  };
+  GemmArgs b = a;
+  void *ca = nullptr, *cb = nullptr, *cc = nullptr, *cp = nullptr, *cbias = nullptr;
+  int rc = kOk, ld = 0;
+  if (fix_a) {
+    const int rows = a.op_a == GINN_HIP_OP_N ? a.m : a.k, cols = a.op_a == GINN_HIP_OP_N ? a.k : a.m;
+    rc = take(a.A, rows, cols, a.lda, true, &ca, &ld);
+    b.A = ca;
+    b.lda = ld;
+  }
+  if (rc == kOk && fix_b) {
+    const int rows = a.op_b == GINN_HIP_OP_N ? a.k : a.n, cols = a.op_b == GINN_HIP_OP_N ? a.n : a.k;
+    rc = take(a.B, rows, cols, a.ldb, true, &cb, &ld);
+    b.B = cb;
+    b.ldb = ld;
+  }
+  if (rc == kOk && fix_c) {
+    // The epilogue reads the old values from the kept pre-activation when there is one, from C otherwise.
+    rc = take(a.C, a.m, a.n, a.ldc, a.beta != 0.f && !a.pre, &cc, &ld);
+    b.C = cc;
+    b.ldc = ld;
+    if (rc == kOk && a.pre) {
+      rc = take(a.pre, a.m, a.n, a.ldc, a.beta != 0.f, &cp, &ld);
+      b.pre = cp;
+    }
+  }
+  if (rc == kOk && fix_bias) {
+    rc = take(a.bias, a.m, 1, a.m, true, &cbias, &ld);
+    b.bias = cbias;
+  }
+  if (rc == kOk) rc = launch_gemm(ctx, b);
+  if (rc == kOk && cc) rc = ginn_hip_copy_2d(ctx, dt, a.m, a.n, cc, b.ldc, a.C, a.ldc, 0);
+  if (rc == kOk && cp) rc = ginn_hip_copy_2d(ctx, dt, a.m, a.n, cp, b.ldc, a.pre, a.ldc, 0);
+  for (int i = 0; i < used; ++i) {
+    const int rc_free = ginn_hip_free(ctx, blocks[i]);
+    if (rc == kOk) rc = rc_free;
+  }
+  return rc;
+}
+
 // Extents that are no multiples of the tuned kernels' tiles (4000^3; m = 1000) left a product on
 // the any-shape kernel, several times slower than its aligned neighbours (fp16 4000^3: 596 us
 // against 112 us for 4096^3).  With leading dimensions and pointers that allow 16-byte accesses the
@@ -60,14 +139,15 @@ int launch_gemm_ragged(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (m0 < 256 || n0 < 256 || k0 < 4 * bk) return kUnsupported;
   // Worth the extra launches: a core of at least 512^3 multiply-adds that is most of the product.  Ragged
   // rows cost more than a ragged K (their few rows times all of K are a slow shape for the any-shape
-  // kernel): only from 4 (fp32) or 8 x as much on, and not for the 16-bit types with a K-contiguous A, where
-  // the any-shape kernel alone is as fast (measured, us before -> after: fp16 NN 4000^3 596 -> 217,
+  // kernel): only from 4 (fp32) or 8 x as much on, and not for the 16-bit types with a K-contiguous A whose K
+  // allows 16-byte loads, where the any-shape kernel alone is as fast (measured, us before -> after: fp16 NN 4000^3 596 -> 217,
   // 2000^3 106 -> 59, 1024 x 1024 x 1000 20.6 -> 11.7; fp32 NN 4000^3 1220 -> 996, 2000^3 242 -> 185,
   // 1000 x 1024 x 1024 42.7 -> 29.8; but fp16 TN 4000^3 239 -> 357, 1000^3 14.6 -> 21.2).
   const double core = static_cast<double>(m0) * n0 * k0, all = static_cast<double>(a.m) * a.n * a.k;
   if (core < 134217728. || core < 0.75 * all) return kUnsupported;
   const bool f32 = a.dtype == GINN_HIP_F32;
-  if (m0 < a.m && (core < (f32 ? 536870912. : 1073741824.) || (!f32 && a.op_a == GINN_HIP_OP_T))) return kUnsupported;
+  if (m0 < a.m && (core < (f32 ? 536870912. : 1073741824.) || (!f32 && a.op_a == GINN_HIP_OP_T && a.k % per16 == 0)))
+    return kUnsupported;
 
   const char* A = static_cast<const char*>(a.A);
   const char* B = static_cast<const char*>(a.B);
@@ -152,6 +232,8 @@ int launch_gemm(ginn_hip_ctx* ctx, const GemmArgs& a) {
   rc = launch_gemm_bsmall(ctx, a);
   if (rc != kUnsupported) return rc;
   rc = launch_gemm_mid(ctx, a);
+  if (rc != kUnsupported) return rc;
+  rc = launch_gemm_realigned(ctx, a);
   if (rc != kUnsupported) return rc;
   rc = launch_gemm_ragged(ctx, a);
   if (rc != kUnsupported) return rc;

@@ -85,6 +85,7 @@ extern "C" int ginn_hip_gemm_noalloc(int device, void* stream, ginn_hip_dtype dt
   local.workspace = st.scratch_ptr;
   local.workspace_bytes = kScratchBytes;
   local.num_cus = st.num_cus;
+  local.may_allocate = false;
   GemmArgs a{};
   a.dtype = dtype;
   a.op_a = op_a;

@@ -188,7 +188,12 @@ int ginn_hip_arena_size(const ginn_hip_arena* arena, size_t* bytes);
 /* C[m x n] = op(A)[m x k] * op(B)[k x n] + beta * C, alpha fixed to 1;
  * replaces gpu_gemm -> cublasSgemm / cublasHgemm (ginn/prod.h:32-66).
  * fp16 / bf16 operands are multiplied exactly and accumulated in fp32; the
- * result is rounded to the storage type once.  beta == 0 never reads C. */
+ * result is rounded to the storage type once (twice where a large product
+ * with extents that are no multiples of the kernels' tiles is cut into a
+ * tuned core and a rest).  beta == 0 never reads C.  A large product whose
+ * leading dimensions or pointers rule out 16-byte accesses is computed on
+ * copies with padded leading dimensions, in blocks of the context's pool
+ * (ginn_hip_malloc / ginn_hip_free); not while the stream is captured. */
 int ginn_hip_gemm(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, ginn_hip_op op_a,
                   ginn_hip_op op_b, int m, int n, int k, const void* A,
                   int lda, const void* B, int ldb, float beta, void* C,

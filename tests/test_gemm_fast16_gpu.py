@@ -352,3 +352,23 @@ def test_ragged_extents_with_aligned_leading_dimensions(dev, dt, op_a, op_b, m, 
     dev.sync()
     err = float((C.double().transpose(1, 2) - want).norm() / want.norm())
     assert err <= 2 * _bound(dt), err
+
+
+@pytest.mark.parametrize("dt", [capi.F32, capi.F16, capi.BF16])
+@pytest.mark.parametrize("op_a,op_b", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(1501, 1503, 1505), (1024, 1024, 1001), (1001, 1024, 1024), (2047, 2049, 515)])
+@pytest.mark.parametrize("beta", [0.0, 0.5])
+def test_odd_leading_dimensions_of_large_products(dev, dt, op_a, op_b, m, n, k, beta):
+    """Leading dimensions that rule out 16-byte accesses (odd row counts): a large product runs on copies
+    with padded leading dimensions from the context's pool (one, two or all three of A, B, C copied; C
+    copied in when beta reads it and always copied back), a smaller one on the any-shape kernel."""
+    from gpu_util import torch_dtype
+    torch = dev.torch
+    A, B, lda, ldb = _operands(dev, dt, op_a, op_b, m, n, k, 1, m + 2 * n + 3 * k)
+    g = torch.Generator(device="cuda").manual_seed(m)
+    C = torch.randn(1, n, m, generator=g, device="cuda").to(torch_dtype(dt))
+    want = _expected(A, B, op_a, op_b) + beta * C.double().transpose(1, 2)
+    dev.gemm(dt, op_a, op_b, m, n, k, A.data_ptr(), lda, B.data_ptr(), ldb, beta, C.data_ptr(), m)
+    dev.sync()
+    err = float((C.double().transpose(1, 2) - want).norm() / want.norm())
+    assert err <= 2 * _bound(dt), err
