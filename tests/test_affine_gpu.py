@@ -79,7 +79,9 @@ def test_reference_affine_goldens(dev, golden, dt):
                                    (10, 64, 512, 0), (256, 256, 128, 64), (512, 2048, 256, 0),
                                    (384, 128, 2048, 0), (3072, 4096, 256, 0), (1024, 1, 384, 0),
                                    (2048, 8, 640, 64), (256, 64, 128, 0), (64, 256, 256, 64), (512, 40, 192, 0),
-                                   (1024, 512, 256, 64)])
+                                   (1024, 512, 256, 64),
+                                   # odd leading dimensions, large: the products run on padded copies
+                                   (1001, 1003, 1005, 0), (1501, 1503, 1505, 515)])
 def test_affine_forward(dev, dt, act, shape):
     """m, n, k, k2 (k2 > 0 adds a second (W, X) pair).  For the 16-bit types the
     aligned shapes take the tuned kernels with their fused epilogues: 128 x 128
