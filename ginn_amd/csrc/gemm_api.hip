@@ -123,8 +123,13 @@ int launch_gemm_realigned(ginn_hip_ctx* ctx, const GemmArgs& a) {
 // around it (any-shape kernel) over the whole K tiles, adding to that, with the caller's epilogue.
 // A 16-bit sum is then rounded to the storage type once in between, as between the (W, X) pairs of
 // an Affine.
-int launch_gemm_ragged(ginn_hip_ctx* ctx, const GemmArgs& a) {
+//
+// The same cut with 256 as the unit, tried before the 128 x 128 kernel takes a 16-bit product whole: extents
+// that are multiples of 128 but not of 256 keep the 256 x 256 kernel for the core when that has the tiles
+// the kernel wants, and leave strips of 128 .. 255 rows / columns to the 128 x 128 kernel.
+int launch_gemm_ragged(ginn_hip_ctx* ctx, const GemmArgs& a, int unit) {
   if (a.batch != 1 || a.acols || a.bcols || a.ccols) return kUnsupported;
+  if (unit == 256 && (a.dtype == GINN_HIP_F32 || a.k < 256)) return kUnsupported;
   const long long es = static_cast<long long>(dtype_size(a.dtype));
   const int per16 = static_cast<int>(16 / es), bk = static_cast<int>(128 / es);
   if (a.lda % per16 || a.ldb % per16 || a.ldc % per16) return kUnsupported;
@@ -132,10 +137,15 @@ int launch_gemm_ragged(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (!aligned16(a.A) || !aligned16(a.B) || !aligned16(a.C) || (a.pre && !aligned16(a.pre)) ||
       (a.bias && !aligned16(a.bias)))
     return kUnsupported;
-  const int m0 = a.m / 128 * 128, k0 = a.k / bk * bk;
-  // With a K-contiguous B the tuned kernels mask a partly filled last tile column themselves.
-  const int n0 = a.op_b == GINN_HIP_OP_N ? a.n : a.n / 128 * 128;
+  const int m0 = a.m / unit * unit, k0 = a.k / bk * bk;
+  // With a K-contiguous B the 128 x 128 kernel masks a partly filled last tile column itself.
+  const int n0 = unit == 128 && a.op_b == GINN_HIP_OP_N ? a.n : a.n / unit * unit;
   if (m0 == a.m && n0 == a.n && k0 == a.k) return kUnsupported;
+  if (unit == 256) {
+    // Only what the 128 x 128 kernel would otherwise take whole, and only for a core the 256 x 256 kernel takes.
+    if (a.m % 128 || a.n % 128 || k0 != a.k) return kUnsupported;
+    if (static_cast<long long>(m0 / 256) * (n0 / 256) * 16 < 9ll * ctx->num_cus) return kUnsupported;
+  }
   if (m0 < 256 || n0 < 256 || k0 < 4 * bk) return kUnsupported;
   // Worth the extra launches: a core of at least 512^3 multiply-adds that is most of the product.  Ragged
   // rows cost more than a ragged K (their few rows times all of K are a slow shape for the any-shape
@@ -144,9 +154,10 @@ int launch_gemm_ragged(ginn_hip_ctx* ctx, const GemmArgs& a) {
   // 2000^3 106 -> 59, 1024 x 1024 x 1000 20.6 -> 11.7; fp32 NN 4000^3 1220 -> 996, 2000^3 242 -> 185,
   // 1000 x 1024 x 1024 42.7 -> 29.8; but fp16 TN 4000^3 239 -> 357, 1000^3 14.6 -> 21.2).
   const double core = static_cast<double>(m0) * n0 * k0, all = static_cast<double>(a.m) * a.n * a.k;
-  if (core < 134217728. || core < 0.75 * all) return kUnsupported;
+  if (core < 134217728. || core < (unit == 256 ? 0.85 : 0.75) * all) return kUnsupported;
   const bool f32 = a.dtype == GINN_HIP_F32;
-  if (m0 < a.m && (core < (f32 ? 536870912. : 1073741824.) || (!f32 && a.op_a == GINN_HIP_OP_T && a.k % per16 == 0)))
+  if (unit == 128 && m0 < a.m &&
+      (core < (f32 ? 536870912. : 1073741824.) || (!f32 && a.op_a == GINN_HIP_OP_T && a.k % per16 == 0)))
     return kUnsupported;
 
   const char* A = static_cast<const char*>(a.A);
@@ -229,13 +240,15 @@ int launch_gemm(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (rc != kUnsupported) return rc;
   rc = launch_gemm_fast16(ctx, a);
   if (rc != kUnsupported) return rc;
+  rc = launch_gemm_ragged(ctx, a, 256);
+  if (rc != kUnsupported) return rc;
   rc = launch_gemm_bsmall(ctx, a);
   if (rc != kUnsupported) return rc;
   rc = launch_gemm_mid(ctx, a);
   if (rc != kUnsupported) return rc;
   rc = launch_gemm_realigned(ctx, a);
   if (rc != kUnsupported) return rc;
-  rc = launch_gemm_ragged(ctx, a);
+  rc = launch_gemm_ragged(ctx, a, 128);
   if (rc != kUnsupported) return rc;
   return launch_gemm_generic(ctx, a);
 }

@@ -336,12 +336,15 @@ def test_seeded_random_shapes(dev, seed):
 @pytest.mark.parametrize("dt", [capi.F32, capi.F16, capi.BF16])
 @pytest.mark.parametrize("op_a,op_b", [(0, 0), (0, 1), (1, 0), (1, 1)])
 @pytest.mark.parametrize("m,n,k", [(1024, 1024, 1000), (2000, 2000, 2000), (1000, 1024, 1024), (1160, 1096, 1032),
-                                   (1024, 520, 4100)])
+                                   (1024, 520, 4100),
+                                   # multiples of 128 but not of 256: 256 x 256 kernel for the core, strips beside it
+                                   (3200, 3200, 320), (3328, 4224, 256)])
 @pytest.mark.parametrize("beta", [0.0, 1.0])
 def test_ragged_extents_with_aligned_leading_dimensions(dev, dt, op_a, op_b, m, n, k, beta):
     """Extents that are no multiples of the tuned kernels' tiles while leading dimensions and pointers
     allow 16-byte accesses: the product is cut into the last K % 64 (32 for fp32) values over the whole
-    output, the aligned core on the tuned kernels, and the ragged rows / columns around it."""
+    output, the aligned core on the tuned kernels, and the ragged rows / columns around it (16-bit extents
+    that are multiples of 128 but not of 256: a core of 256-multiples and strips of 128)."""
     from gpu_util import torch_dtype
     torch = dev.torch
     A, B, lda, ldb = _operands(dev, dt, op_a, op_b, m, n, k, 1, m + n + k)
