@@ -67,42 +67,59 @@ int launch_gemm_realigned(ginn_hip_ctx* ctx, const GemmArgs& a) {
   const ginn_hip_dtype dt = static_cast<ginn_hip_dtype>(a.dtype);
   void* blocks[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
   int used = 0;
-  auto padded = [](int rows) { return (rows + 63) / 64 * 64; };
-  // A copy of the stored rows x cols matrix at src with a padded leading dimension (filled when `fill`).
-  auto take = [&](const void* src, int rows, int cols, int ld, bool fill, void** out, int* ld_out) {
-    *ld_out = padded(rows);
-    int rc = ginn_hip_malloc(ctx, static_cast<size_t>(*ld_out) * cols * es, out);
+  // When all three matrices of a 16-bit product are copied anyway, the copies are zero-padded to whole tiles
+  // as well (rows and columns to multiples of 128, K to the K tile): the tuned kernels then take the product
+  // whole, where the ragged rows and columns of 4095 x 4097 x 4099 cost the any-shape kernel more than the
+  // core costs (435 -> 212 us; 2047 x 2049 x 2051 106 -> 76 us).  fp32 keeps its extents (the same padding
+  // there: 1311 -> 1366 us and 228 -> 298 us).
+  const bool whole_tiles = fix_a && fix_b && fix_c && a.dtype != GINN_HIP_F32;
+  const int bk = static_cast<int>(128 / es);
+  auto up = [](int v, int unit) { return (v + unit - 1) / unit * unit; };
+  const int mp = whole_tiles ? up(a.m, 128) : a.m, np = whole_tiles ? up(a.n, 128) : a.n;
+  const int kp = whole_tiles ? up(a.k, bk) : a.k;
+  // A block for a stored rows_p x cols_p matrix with a padded leading dimension, zeroed when larger than the
+  // rows x cols matrix at src, which is copied in when `fill`.
+  auto take = [&](const void* src, int rows, int cols, int ld, int rows_p, int cols_p, bool fill, void** out,
+                  int* ld_out) {
+    *ld_out = up(rows_p, 64);
+    const size_t bytes = static_cast<size_t>(*ld_out) * cols_p * es;
+    int rc = ginn_hip_malloc(ctx, bytes, out);
     if (rc != kOk) return rc;
     blocks[used++] = *out;
-    return fill ? ginn_hip_copy_2d(ctx, dt, rows, cols, src, ld, *out, *ld_out, 0) : kOk;
+    if (rows_p != rows || cols_p != cols) rc = ginn_hip_memset(ctx, *out, 0, bytes);
+    if (rc == kOk && fill) rc = ginn_hip_copy_2d(ctx, dt, rows, cols, src, ld, *out, *ld_out, 0);
+    return rc;
   };
   GemmArgs b = a;
+  b.m = mp;
+  b.n = np;
+  b.k = kp;
   void *ca = nullptr, *cb = nullptr, *cc = nullptr, *cp = nullptr, *cbias = nullptr;
   int rc = kOk, ld = 0;
   if (fix_a) {
-    const int rows = a.op_a == GINN_HIP_OP_N ? a.m : a.k, cols = a.op_a == GINN_HIP_OP_N ? a.k : a.m;
-    rc = take(a.A, rows, cols, a.lda, true, &ca, &ld);
+    const bool an = a.op_a == GINN_HIP_OP_N;
+    rc = take(a.A, an ? a.m : a.k, an ? a.k : a.m, a.lda, an ? mp : kp, an ? kp : mp, true, &ca, &ld);
     b.A = ca;
     b.lda = ld;
   }
   if (rc == kOk && fix_b) {
-    const int rows = a.op_b == GINN_HIP_OP_N ? a.k : a.n, cols = a.op_b == GINN_HIP_OP_N ? a.n : a.k;
-    rc = take(a.B, rows, cols, a.ldb, true, &cb, &ld);
+    const bool bn = a.op_b == GINN_HIP_OP_N;
+    rc = take(a.B, bn ? a.k : a.n, bn ? a.n : a.k, a.ldb, bn ? kp : np, bn ? np : kp, true, &cb, &ld);
     b.B = cb;
     b.ldb = ld;
   }
   if (rc == kOk && fix_c) {
     // The epilogue reads the old values from the kept pre-activation when there is one, from C otherwise.
-    rc = take(a.C, a.m, a.n, a.ldc, a.beta != 0.f && !a.pre, &cc, &ld);
+    rc = take(a.C, a.m, a.n, a.ldc, mp, np, a.beta != 0.f && !a.pre, &cc, &ld);
     b.C = cc;
     b.ldc = ld;
     if (rc == kOk && a.pre) {
-      rc = take(a.pre, a.m, a.n, a.ldc, a.beta != 0.f, &cp, &ld);
+      rc = take(a.pre, a.m, a.n, a.ldc, mp, np, a.beta != 0.f, &cp, &ld);
       b.pre = cp;
     }
   }
-  if (rc == kOk && fix_bias) {
-    rc = take(a.bias, a.m, 1, a.m, true, &cbias, &ld);
+  if (rc == kOk && a.bias && (fix_bias || mp != a.m)) {
+    rc = take(a.bias, a.m, 1, a.m, mp, 1, true, &cbias, &ld);
     b.bias = cbias;
   }
   if (rc == kOk) rc = launch_gemm(ctx, b);
