@@ -51,11 +51,11 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
       // and no partial tiles to fold in a second launch (which costs what
       // some 20 K tiles of such a workgroup cost: the fewer the tiles, the
       // shorter the K up to which that holds).
-      const long long tiles64 = (long long)(a.m / 64) * (a.n / 64) * a.batch;
+      const long long tiles64 = (long long)(a.m / 64) * ((a.n + 63) / 64) * a.batch;
       const int kt = a.k / bk;
       const bool enough = tiles64 >= ctx->num_cus || (tiles64 * 4 >= 3 * ctx->num_cus && kt <= 64) ||
                           (tiles64 * 8 >= 3 * ctx->num_cus && kt <= 32);
-      if (a.m % 64 == 0 && a.n % 64 == 0 && enough && tiles64 <= 2 * ctx->num_cus)
+      if (a.m % 64 == 0 && (a.n % 64 == 0 || any_n) && enough && tiles64 <= 2 * ctx->num_cus)
         fm = 1, fn = 1, f32_tiny_tiles = true;
       else if (fm == 2 && fn == 2) fn = 1;
       const long long tiles = (long long)(a.m / (64 * fm)) * ((a.n + 64 * fn - 1) / (64 * fn)) * a.batch;
