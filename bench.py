@@ -175,11 +175,11 @@ def bench_mlp(iters, cpu, executor=6):
     executor: 0 = Graph (node by node), 2 = level executor, 6 = level executor frozen after its first pass,
     14 = the frozen pass recorded as a device graph."""
     import numpy as np
-    from oracle import nodes as N
+    from ginn_amd import capi
     ex = _examples()
     ex.scenario_set_executor(executor)
     rng = np.random.default_rng(1)
-    dims, acts, batch = [784, 512, 512, 10], [N.TANH, N.RELU, N.IDENTITY], 64
+    dims, acts, batch = [784, 512, 512, 10], [capi.ACT_TANH, capi.ACT_RELU, capi.ACT_IDENTITY], 64
     x = _f32(rng.uniform(0, 1, (dims[0], batch)))
     labels = rng.integers(0, 10, batch).astype(np.int32)
     Ws = [_f32(_xavier(rng, dims[i + 1], dims[i])) for i in range(3)]
@@ -194,9 +194,19 @@ def bench_mlp(iters, cpu, executor=6):
         raise SystemExit(ex.scenario_last_error().decode())
     flops = 3 * sum(2.0 * dims[i + 1] * dims[i] * batch for i in range(3)) - 2.0 * 512 * 784 * batch
     ex.scenario_set_executor(0)
+    # Algorithmic bytes of the pass: 4 (M K + K N + M N (1 + beta)) over its eight products (three forward,
+    # three dW = dpre X^T, two dX = W^T dpre: the input takes no gradient), beta = 0 throughout.
+    by = 0.0
+    for i in range(3):
+        mm, kk = dims[i + 1], dims[i]
+        per = 4.0 * (mm * kk + kk * batch + mm * batch)
+        by += per * (3 if i else 2)
     r = {"config": f"mlp fp32 b64 784-512-512-10 fwd+bwd, executor={executor}", "gpu_ms": round(ms.value, 4),
-         "gflops": round(flops / ms.value / 1e6, 1)}
+         "gflops": round(flops / ms.value / 1e6, 1), "gbs": round(by / ms.value / 1e6, 1), "algorithmic_bytes": int(by)}
+    if executor & 8:
+        r["kernels_per_pass"] = int(ex.scenario_recorded_kernels())
     if cpu:
+        from oracle import nodes as N
         r["cpu_ms"] = round(_cpu_timed(lambda: N.mlp_forward_backward(acts, Ws, bs, x, labels)), 3)
         r["cpu"] = "oracle (numpy fp32 restatement), 1 thread"
     return r
@@ -213,7 +223,6 @@ def bench_lstm(iters, cpu, mode=7, gather=False):
     group into one GatherProd (right operands read, and their gradients added,
     where they are) instead of RowwiseCat + Prod + RowwiseUncat."""
     import numpy as np
-    from oracle import nodes as N
     ex = _examples()
     ex.scenario_set_autobatch_gather(1 if gather else 0)
     rng = np.random.default_rng(2024)
@@ -235,13 +244,23 @@ def bench_lstm(iters, cpu, mode=7, gather=False):
     if rc:
         raise SystemExit(ex.scenario_last_error().decode())
     flops = 3 * 2.0 * 4 * H * (E + H) * total
+    # Algorithmic bytes of the pass: per time step t with n_t sequences alive, the merged products
+    # Z = W X_t and dX_t = W^T dZ_t (4 (M K + K n_t + M n_t) each), and once the weight gradient over all
+    # columns (4 (M total + K total + M K)).
+    M_, K_ = 4 * H, E + H
+    alive = [sum(1 for L in lens if L > t) for t in range(max(lens))]
+    by = sum(2 * 4.0 * (M_ * K_ + K_ * n_t + M_ * n_t) for n_t in alive) + 4.0 * (M_ * total + K_ * total + M_ * K_)
     r = {"config": f"lstm gates fp32 256 seqs (sum len {total}) E128 H256 fwd+bwd, autobatch={('gather' if gather else 'cat') if mode & 1 else 0}, "
                    f"level executor={(mode >> 1) & 1}, frozen={(mode >> 2) & 1}, device graph={(mode >> 3) & 1}, "
                    f"chains={(mode >> 4) & 1}",
          "gpu_ms": round(ms.value, 3), "gflops": round(flops / ms.value / 1e6, 1), "graph_nodes": nodes.value,
          "products": prods.value, "table_launches_per_pass": launches.value,
-         "first_pass_ms": round(first_ms.value, 2)}
+         "first_pass_ms": round(first_ms.value, 2), "gbs": round(by / ms.value / 1e6, 1),
+         "algorithmic_bytes": int(by)}
+    if mode & 8:
+        r["kernels_per_pass"] = int(ex.scenario_recorded_kernels())
     if cpu:
+        from oracle import nodes as N
         offs = np.concatenate([[0], np.cumsum(lens)])
         xl = [np.asfortranarray(xs[:, offs[s]:offs[s + 1]]) for s in range(nseq)]
         r["cpu_ms"] = round(_cpu_timed(lambda: N.lstm_backward(W, b, xl, mask)), 2)
@@ -298,6 +317,22 @@ def bench_attention(h, steps, warmup, cpu):
             r["cpu"] = "oracle_bgemm_f32, 1 thread"
         out.append(r)
     return out
+
+
+def time_product(h, dtype, layout, m, n, k, steps, warmup):
+    """Milliseconds per product (HIP events on the context's stream around back-to-back launches issued from
+    native code, so that launches of a few microseconds are not bound by the interpreter); goes through
+    ginn_hip_gemm_strided_batched with one slice, which selects kernels exactly as ginn_hip_gemm does."""
+    A, B, C, lda, ldb = h.operands(dtype, layout, m, n, k)
+    ex = _examples()
+    ms = c_float(0)
+    args = (h.ctx, DT[dtype], int(layout[0] == "T"), int(layout[1] == "T"), m, n, k, c_void_p(A.data_ptr()), lda,
+            ctypes.c_longlong(0), c_void_p(B.data_ptr()), ldb, ctypes.c_longlong(0), c_float(0.0),
+            c_void_p(C.data_ptr()), m, ctypes.c_longlong(0), 1)
+    for _ in range(2):  # the second measurement counts: the first meets clocks that are still moving
+        if ex.scenario_time_batched_gemm(*args, warmup, steps, byref(ms)) != 0:
+            raise SystemExit(f"scenario_time_batched_gemm: {ex.scenario_last_error().decode()}")
+    return ms.value
 
 
 def bench_update(h, steps, warmup, cpu):
@@ -366,7 +401,7 @@ def bench_gpt(iters, cpu, dtype="bf16", executor=6, train=None):
     14 = the frozen pass recorded as a device graph.  train: None, or "adam" / "sgd": every pass
     ends with the update of all 20 weights (one launch), i.e. a whole training step is timed."""
     import numpy as np
-    from oracle import nodes as N
+    from ginn_amd import capi
     ex = _examples()
     ex.scenario_set_executor(executor)
     ex.scenario_set_training({None: -1, "sgd": 0, "adam": 1}[train], ctypes.c_float(1e-4), ctypes.c_float(5.0))
@@ -378,7 +413,7 @@ def bench_gpt(iters, cpu, dtype="bf16", executor=6, train=None):
     params = {k: _f32(rng.standard_normal(s) * 0.02) for k, s in shapes.items()}
     x = _f32(rng.standard_normal((C, B, T)))
     targets = rng.integers(0, V, B * T).astype(np.int32)
-    pin = [params[k] for k in N.GptBlockParams.NAMES]
+    pin = [params[k] for k in capi.GPT_PARAM_NAMES]
     grads = [np.zeros_like(a) for a in pin]
     dx, loss = np.zeros_like(x), np.zeros(1, np.float32)
     ms, nodes = ctypes.c_float(0), ctypes.c_int(0)
@@ -396,6 +431,7 @@ def bench_gpt(iters, cpu, dtype="bf16", executor=6, train=None):
          "gpu_ms": round(ms.value, 3), "tflops": round(3 * fwd / ms.value / 1e9, 1), "graph_nodes": nodes.value,
          "loss": round(float(loss[0]), 4)}
     if cpu:
+        from oracle import nodes as N
         p = N.GptBlockParams(**params)
         r["cpu_ms"] = round(_cpu_timed(lambda: N.gpt_layer_forward_backward(p, x, targets, nh)), 1)
         r["cpu"] = "oracle (numpy fp32 restatement, BLAS products), 1 thread"
@@ -443,24 +479,51 @@ def measured_traffic(dtype, layout, m, n, k):
     return None, None
 
 
-def other_configs(cpu):
-    """The graph-level configurations of the build target, a few passes each, outside the headline's timed
-    region: GPU ms per fwd+bwd pass through the frozen level executor, and the CPU oracle on one thread."""
+def other_configs(h, cpu):
+    """The other configurations of the build target, outside the headline's timed region.  Graph level (GPU
+    ms per fwd+bwd pass through the frozen level executor, algorithmic GB/s, kernel launches per pass counted
+    in a recording of the pass, the CPU oracle on one thread beside them): min-GPT layer, MLP, autobatched
+    LSTM.  Kernel level: the six attention products, the skinny shapes M = K = 4096 and two more squares of
+    the GEMM sweep, each against the roofline that bounds it."""
     out = {}
     g = bench_gpt(30, cpu, executor=6)
     out["gpt_ms"], out["gpt_tflops"] = g["gpu_ms"], g["tflops"]
     if cpu:
         out["gpt_cpu_ms"] = g["cpu_ms"]
     r = bench_mlp(100, cpu, executor=6)
-    out["mlp_ms"] = r["gpu_ms"]
+    out["mlp_ms"], out["mlp_gbs"] = r["gpu_ms"], r["gbs"]
     if cpu:
         out["mlp_cpu_ms"] = r["cpu_ms"]
+    out["mlp_kernels_per_pass"] = bench_mlp(2, False, executor=14)["kernels_per_pass"]
     r = bench_lstm(10, cpu, mode=23, gather=True)
-    out["lstm_ms"] = r["gpu_ms"]
+    out["lstm_ms"], out["lstm_gbs"] = r["gpu_ms"], r["gbs"]
+    out["lstm_table_launches_per_pass"] = r["table_launches_per_pass"]
     if cpu:
         out["lstm_cpu_ms"] = r["cpu_ms"]
+    out["lstm_kernels_per_pass"] = bench_lstm(2, False, mode=31, gather=True)["kernels_per_pass"]
+    out["attention"] = {r["config"].split("batch 128 ")[1]: {"us": round(r["gpu_ms"] * 1e3, 2), "gbs": r["gbs"],
+                                                             "frac_hbm": r["frac_hbm"], "tflops": r["tflops"]}
+                        for r in bench_attention(h, 200, 20, False)}
+    skinny = {}
+    for dt in ("f32", "f16"):
+        for nn in (1, 16, 64):
+            ms = time_product(h, dt, "NN", 4096, nn, 4096, 200, 20)
+            by = ESIZE[dt] * (4096 * 4096 + 4096 * nn + 4096 * nn)
+            skinny[f"{dt}_n{nn}"] = {"us": round(ms * 1e3, 2), "gbs": round(by / ms / 1e6, 1),
+                                     "frac_hbm": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    out["skinny_m4096_k4096"] = skinny
+    squares = {}
+    for size, steps in ((4096, 100), (2048, 200)):
+        ms = time_product(h, "f16", "NN", size, size, size, steps, 20)
+        tf = 2.0 * size ** 3 / ms / 1e9
+        squares[f"f16_NN_{size}"] = {"us": round(ms * 1e3, 2), "tflops": round(tf, 1),
+                                     "frac_mfma": round(tf / PEAK_TFLOPS["f16"], 4)}
+    out["squares"] = squares
     out["note"] = ("fwd+bwd per pass: min-GPT layer bf16 (d768 h12 T512 B8 ff3072 V8192), MLP fp32 b64 784-512-512-10, "
-                   "autobatched LSTM fp32 256 seqs; cpu = numpy fp32 oracle on 1 thread")
+                   "autobatched LSTM fp32 256 seqs; gbs = algorithmic bytes of the pass's products per second; "
+                   "kernels_per_pass = kernel nodes of the pass recorded as a device graph; attention = fp16 batch 128 "
+                   "products, skinny = M = K = 4096 NN with the split-K fold included, against 8 TB/s; squares "
+                   "against 2.5 PFLOP/s; cpu = numpy fp32 oracle on 1 thread")
     return out
 
 
@@ -592,7 +655,7 @@ def main():
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(m, k, min(a.cpu_panel, n), a.dtype)
     if not a.no_configs:
-        line["configs"] = other_configs(not a.no_cpu)
+        line["configs"] = other_configs(h, not a.no_cpu)
     print(json.dumps(line), flush=True)
 
 

@@ -20,6 +20,11 @@ OP_N, OP_T = 0, 1
  ACT_SOFTMAX, ACT_LOG, ACT_SQRT) = range(9)
 
 # name -> (restype, argtypes); mirrors include/ginn_hip.h one to one.
+# Order in which scenario_gpt_layer (ginn_amd/examples/configs.cpp) takes the 20 parameters of one
+# decoder layer + final LayerNorm + vocabulary head (examples/min-gpt.cu.cpp:93-163, 227-260).
+GPT_PARAM_NAMES = ["ln1_g", "ln1_b", "Wk", "bk", "Wq", "bq", "Wv", "bv", "Wp", "bp", "ln2_g", "ln2_b", "W1", "b1",
+                   "W2", "b2", "lnf_g", "lnf_b", "Wh", "bh"]
+
 PROTOTYPES = {
     "ginn_hip_last_error": (c_char_p, []),
     "ginn_hip_version": (c_char_p, []),
@@ -34,6 +39,7 @@ PROTOTYPES = {
     "ginn_hip_free": (c_int, [c_void_p, c_void_p]),
     "ginn_hip_pool_configure": (c_int, [c_void_p, c_int, c_size_t]),
     "ginn_hip_pool_trim": (c_int, [c_void_p]),
+    "ginn_hip_gemm_temp_budget": (c_int, [c_void_p, c_size_t]),
     "ginn_hip_pool_stats": (c_int, [c_void_p, POINTER(c_size_t), POINTER(c_size_t)]),
     "ginn_hip_memcpy_h2d": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "ginn_hip_memcpy_d2h": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
@@ -140,6 +146,7 @@ PROTOTYPES = {
     "ginn_hip_capture_begin": (c_int, [c_void_p]),
     "ginn_hip_capture_end": (c_int, [c_void_p, POINTER(c_void_p)]),
     "ginn_hip_graph_launch": (c_int, [c_void_p]),
+    "ginn_hip_graph_kernel_count": (c_int, [c_void_p, POINTER(c_size_t)]),
     "ginn_hip_graph_destroy": (c_int, [c_void_p]),
     "ginn_hip_event_record": (c_int, [c_void_p, c_int]),
     "ginn_hip_event_elapsed_ms": (c_int, [c_void_p, c_int, c_int, POINTER(c_float)]),

@@ -110,6 +110,7 @@ struct ginn_hip_ctx {
   hipEvent_t events[64] = {};
   int num_cus = 256;
   bool may_allocate = true;  // false for the stack context of the entry point that must not allocate
+  size_t gemm_temp_budget = size_t(2) << 30;  // ginn_hip_gemm_temp_budget
   ginn_hip_pool pool;
   ginn_hip_fold_queue folds;  // guarded by `mutex`
 };

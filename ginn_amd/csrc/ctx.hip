@@ -7,6 +7,8 @@
 #include <cstdlib>
 #include <iterator>
 
+#include <vector>
+
 #include "common.h"
 
 namespace ginn_hip {
@@ -369,6 +371,13 @@ int ginn_hip_pool_configure(ginn_hip_ctx* ctx, int enabled, size_t limit_bytes) 
   return kOk;
 }
 
+int ginn_hip_gemm_temp_budget(ginn_hip_ctx* ctx, size_t bytes) {
+  GH_CHECK_ARG(ctx, "ginn_hip_gemm_temp_budget: ctx is NULL");
+  std::lock_guard<std::mutex> lock(ctx->mutex);
+  ctx->gemm_temp_budget = bytes;
+  return kOk;
+}
+
 int ginn_hip_pool_trim(ginn_hip_ctx* ctx) {
   GH_CHECK_ARG(ctx, "ginn_hip_pool_trim: ctx is NULL");
   GH_HIP(hipSetDevice(ctx->device));
@@ -571,6 +580,21 @@ int ginn_hip_graph_launch(ginn_hip_graph* graph) {
   GH_CHECK_ARG(graph && graph->exec, "ginn_hip_graph_launch: graph is NULL");
   GH_HIP(hipSetDevice(graph->ctx->device));
   GH_HIP(hipGraphLaunch(graph->exec, graph->ctx->stream));
+  return kOk;
+}
+
+int ginn_hip_graph_kernel_count(ginn_hip_graph* graph, size_t* kernels) {
+  GH_CHECK_ARG(graph && graph->graph && kernels, "ginn_hip_graph_kernel_count: NULL argument");
+  *kernels = 0;
+  size_t n = 0;
+  GH_HIP(hipGraphGetNodes(graph->graph, nullptr, &n));
+  std::vector<hipGraphNode_t> nodes(n);
+  if (n) GH_HIP(hipGraphGetNodes(graph->graph, nodes.data(), &n));
+  for (size_t i = 0; i < n; ++i) {
+    hipGraphNodeType type;
+    GH_HIP(hipGraphNodeGetType(nodes[i], &type));
+    if (type == hipGraphNodeTypeKernel) ++*kernels;
+  }
   return kOk;
 }
 

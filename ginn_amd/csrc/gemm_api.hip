@@ -70,8 +70,6 @@ int launch_gemm_realigned(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (capturing != hipStreamCaptureStatusNone) return kUnsupported;
 
   const ginn_hip_dtype dt = static_cast<ginn_hip_dtype>(a.dtype);
-  void* blocks[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
-  int used = 0;
   // When all three matrices of a 16-bit product are copied anyway, the copies are zero-padded to whole tiles
   // as well (rows and columns to multiples of 128, K to the K tile): the tuned kernels then take the product
   // whole, where the ragged rows and columns of 4095 x 4097 x 4099 cost the any-shape kernel more than the
@@ -82,56 +80,82 @@ int launch_gemm_realigned(ginn_hip_ctx* ctx, const GemmArgs& a) {
   auto up = [](int v, int unit) { return (v + unit - 1) / unit * unit; };
   const int mp = whole_tiles ? up(a.m, 128) : a.m, np = whole_tiles ? up(a.n, 128) : a.n;
   const int kp = whole_tiles ? up(a.k, bk) : a.k;
-  // A block for a stored rows_p x cols_p matrix with a padded leading dimension, zeroed when larger than the
+  // A copy: a stored rows_p x cols_p matrix with a padded leading dimension, zeroed when larger than the
   // rows x cols matrix at src, which is copied in when `fill`.
-  auto take = [&](const void* src, int rows, int cols, int ld, int rows_p, int cols_p, bool fill, void** out,
-                  int* ld_out) {
-    *ld_out = up(rows_p, 64);
-    const size_t bytes = static_cast<size_t>(*ld_out) * cols_p * es;
-    int rc = ginn_hip_malloc(ctx, bytes, out);
-    if (rc != kOk) return rc;
-    blocks[used++] = *out;
-    if (rows_p != rows || cols_p != cols) rc = ginn_hip_memset(ctx, *out, 0, bytes);
-    if (rc == kOk && fill) rc = ginn_hip_copy_2d(ctx, dt, rows, cols, src, ld, *out, *ld_out, 0);
-    return rc;
+  struct Copy {
+    const void* src = nullptr;
+    int rows = 0, cols = 0, ld_src = 0, rows_p = 0, cols_p = 0, ld = 0;
+    bool fill = false;
+    void* block = nullptr;
+    size_t bytes = 0;
   };
+  Copy copies_[5];
+  int used = 0;
+  auto plan = [&](const void* src, int rows, int cols, int ld_src, int rows_p, int cols_p, bool fill) {
+    Copy& c = copies_[used];
+    c.src = src;
+    c.rows = rows;
+    c.cols = cols;
+    c.ld_src = ld_src;
+    c.rows_p = rows_p;
+    c.cols_p = cols_p;
+    c.ld = up(rows_p, 64);
+    c.fill = fill;
+    c.bytes = static_cast<size_t>(c.ld) * cols_p * es;
+    return used++;
+  };
+  const bool an = a.op_a == GINN_HIP_OP_N, bn = a.op_b == GINN_HIP_OP_N;
+  int ia = -1, ib = -1, ic = -1, ip = -1, ibias = -1;
+  if (fix_a) ia = plan(a.A, an ? a.m : a.k, an ? a.k : a.m, a.lda, an ? mp : kp, an ? kp : mp, true);
+  if (fix_b) ib = plan(a.B, bn ? a.k : a.n, bn ? a.n : a.k, a.ldb, bn ? kp : np, bn ? np : kp, true);
+  if (fix_c) {
+    // The epilogue reads the old values from the kept pre-activation when there is one, from C otherwise.
+    ic = plan(a.C, a.m, a.n, a.ldc, mp, np, a.beta != 0.f && !a.pre);
+    if (a.pre) ip = plan(a.pre, a.m, a.n, a.ldc, mp, np, a.beta != 0.f);
+  }
+  if (a.bias && (fix_bias || mp != a.m)) ibias = plan(a.bias, a.m, 1, a.m, mp, 1, true);
+  // All blocks first, before anything is written: when the device (or the budget for temporaries) has no
+  // room for them the product still runs where it is, on the any-shape kernels, as it did before this
+  // path existed.  Nothing of C or the kept pre-activation has been touched at that point.
+  size_t total = 0;
+  for (int i = 0; i < used; ++i) total += copies_[i].bytes;
+  if (total > ctx->gemm_temp_budget) return kUnsupported;
+  for (int i = 0; i < used; ++i) {
+    if (ginn_hip_malloc(ctx, copies_[i].bytes, &copies_[i].block) != kOk) {
+      for (int j = 0; j < i; ++j) (void)ginn_hip_free(ctx, copies_[j].block);
+      clear_error();
+      return kUnsupported;
+    }
+  }
+  int rc = kOk;
+  for (int i = 0; i < used && rc == kOk; ++i) {
+    const Copy& c = copies_[i];
+    if (c.rows_p != c.rows || c.cols_p != c.cols) rc = ginn_hip_memset(ctx, c.block, 0, c.bytes);
+    if (rc == kOk && c.fill) rc = ginn_hip_copy_2d(ctx, dt, c.rows, c.cols, c.src, c.ld_src, c.block, c.ld, 0);
+  }
   GemmArgs b = a;
   b.m = mp;
   b.n = np;
   b.k = kp;
-  void *ca = nullptr, *cb = nullptr, *cc = nullptr, *cp = nullptr, *cbias = nullptr;
-  int rc = kOk, ld = 0;
-  if (fix_a) {
-    const bool an = a.op_a == GINN_HIP_OP_N;
-    rc = take(a.A, an ? a.m : a.k, an ? a.k : a.m, a.lda, an ? mp : kp, an ? kp : mp, true, &ca, &ld);
-    b.A = ca;
-    b.lda = ld;
+  if (ia >= 0) {
+    b.A = copies_[ia].block;
+    b.lda = copies_[ia].ld;
   }
-  if (rc == kOk && fix_b) {
-    const bool bn = a.op_b == GINN_HIP_OP_N;
-    rc = take(a.B, bn ? a.k : a.n, bn ? a.n : a.k, a.ldb, bn ? kp : np, bn ? np : kp, true, &cb, &ld);
-    b.B = cb;
-    b.ldb = ld;
+  if (ib >= 0) {
+    b.B = copies_[ib].block;
+    b.ldb = copies_[ib].ld;
   }
-  if (rc == kOk && fix_c) {
-    // The epilogue reads the old values from the kept pre-activation when there is one, from C otherwise.
-    rc = take(a.C, a.m, a.n, a.ldc, mp, np, a.beta != 0.f && !a.pre, &cc, &ld);
-    b.C = cc;
-    b.ldc = ld;
-    if (rc == kOk && a.pre) {
-      rc = take(a.pre, a.m, a.n, a.ldc, mp, np, a.beta != 0.f, &cp, &ld);
-      b.pre = cp;
-    }
+  if (ic >= 0) {
+    b.C = copies_[ic].block;
+    b.ldc = copies_[ic].ld;
   }
-  if (rc == kOk && a.bias && (fix_bias || mp != a.m)) {
-    rc = take(a.bias, a.m, 1, a.m, mp, 1, true, &cbias, &ld);
-    b.bias = cbias;
-  }
+  if (ip >= 0) b.pre = copies_[ip].block;
+  if (ibias >= 0) b.bias = copies_[ibias].block;
   if (rc == kOk) rc = launch_gemm(ctx, b);
-  if (rc == kOk && cc) rc = ginn_hip_copy_2d(ctx, dt, a.m, a.n, cc, b.ldc, a.C, a.ldc, 0);
-  if (rc == kOk && cp) rc = ginn_hip_copy_2d(ctx, dt, a.m, a.n, cp, b.ldc, a.pre, a.ldc, 0);
+  if (rc == kOk && ic >= 0) rc = ginn_hip_copy_2d(ctx, dt, a.m, a.n, b.C, b.ldc, a.C, a.ldc, 0);
+  if (rc == kOk && ip >= 0) rc = ginn_hip_copy_2d(ctx, dt, a.m, a.n, b.pre, b.ldc, a.pre, a.ldc, 0);
   for (int i = 0; i < used; ++i) {
-    const int rc_free = ginn_hip_free(ctx, blocks[i]);
+    const int rc_free = ginn_hip_free(ctx, copies_[i].block);
     if (rc == kOk) rc = rc_free;
   }
   return rc;

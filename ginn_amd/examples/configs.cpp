@@ -144,6 +144,8 @@ int g_exec_mode = 0;
 // gradient that reset_grad() had only flagged was read or added to before its
 // user overwrote it.  None are expected; each is a launch of its own.
 long g_timed_fills = 0;
+// Kernel launches of the pass last recorded as a device graph (forward, reset_grad, backward).
+long g_recorded_kernels = 0;
 
 struct FillCount {
   size_t before = internal::lazy_grad_settles();
@@ -161,6 +163,7 @@ double run_warm(Graph& g, int iters) {
     if ((g_exec_mode & 20) == 20) ex.fuse();
     if ((g_exec_mode & 12) == 12) {
       ex.record_pass();
+      g_recorded_kernels = static_cast<long>(ex.recorded_kernels());
       ex.replay_pass();  // the first replay also loads the graph onto the device
       count.start();
       return run_replays(ex, iters);
@@ -389,6 +392,7 @@ int lstm(int mode, int nseq, const int* lens, int E, int H, const float* W, cons
     }
     if ((mode & 12) == 12) {       // ... as one recorded device graph
       ex.record_pass();
+      g_recorded_kernels = static_cast<long>(ex.recorded_kernels());
       ex.replay_pass();
       FillCount count;
       ms = run_replays(ex, iters);
@@ -500,6 +504,9 @@ const char* scenario_last_error() { return g_error.c_str(); }
 
 // Zero fills on demand during the timed passes of the last scenario (see g_timed_fills).
 long scenario_timed_fills() { return g_timed_fills; }
+// Kernel launches per pass (forward + reset_grad + backward) of the last scenario that was recorded
+// as a device graph (executor mode with bit 3).
+long scenario_recorded_kernels() { return g_recorded_kernels; }
 
 // Columns summed so far by products that waited for the end of their backward pass
 // (internal::LateOuterSum in ginn/node/prod.h).

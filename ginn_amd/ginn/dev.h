@@ -132,7 +132,16 @@ class ContextTable {
   ginn_hip_ctx*& at(size_t idx) {
     GINN_ASSERT(idx < ctx_.size(),
                 "no GPU with index " + std::to_string(idx) + " (" + std::to_string(ctx_.size()) + " visible)");
-    if (!ctx_[idx]) GINN_HIP_CALL(ginn_hip_ctx_create(static_cast<int>(idx), 0, &ctx_[idx]));
+    // Created once, whichever host threads ask first (the reference's multi-threaded
+    // training makes its devices per thread, examples/mnist-dp.cu:158-172).
+    if (!__atomic_load_n(&ctx_[idx], __ATOMIC_ACQUIRE)) {
+      std::lock_guard<std::mutex> lock(mutex_);
+      if (!ctx_[idx]) {
+        ginn_hip_ctx* made = nullptr;
+        GINN_HIP_CALL(ginn_hip_ctx_create(static_cast<int>(idx), 0, &made));
+        __atomic_store_n(&ctx_[idx], made, __ATOMIC_RELEASE);
+      }
+    }
     return ctx_[idx];
   }
   ginn_hip_ctx* beside(size_t idx) {

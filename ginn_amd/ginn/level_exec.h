@@ -101,6 +101,8 @@ class LevelExecutor {
   bool fused_ready_ = false;
 
   std::vector<BaseNodePtr> list_;               // graph order (inputs first)
+  uint64_t id_ = BaseNode::new_epoch();         // names this executor's passes (internal::BesidePass)
+  std::vector<PendingInPlace*> pending_steps_;  // nodes that may postpone their work past their forward()
   std::vector<std::vector<BaseNode*>> levels_;  // by height, ascending
   DevPtr dev_;
   ginn_hip_ctx* ctx_ = nullptr;
@@ -712,6 +714,8 @@ class LevelExecutor {
       if (n->dev() && n->dev()->kind() == GPU) dev_ = n->dev();
     GINN_ASSERT(static_cast<bool>(dev_), "LevelExecutor: no node of the graph lives on a GPU");
     ctx_ = hip_ctx(static_cast<int>(dev_->id().idx));
+    for (auto& n : list_)
+      if (auto* p = dynamic_cast<PendingInPlace*>(n.get())) pending_steps_.push_back(p);
     build_levels();
   }
   LevelExecutor(const LevelExecutor&) = delete;
@@ -802,6 +806,12 @@ class LevelExecutor {
     return *this;
   }
   bool recorded() const { return pass_graph_ != nullptr; }
+  // Kernel launches in the recorded pass (0 before record_pass()).
+  size_t recorded_kernels() const {
+    size_t n = 0;
+    if (pass_graph_) GINN_HIP_CALL(ginn_hip_graph_kernel_count(pass_graph_, &n));
+    return n;
+  }
 
   LevelExecutor& reset_forwarded() {
     if (frozen_) return *this;  // forward() re-runs what it has to
@@ -809,9 +819,12 @@ class LevelExecutor {
     return *this;
   }
 
+  // An in-place step that nobody has asked for by the end of the pass runs
+  // then (PendingInPlace), as at the end of Graph::forward().
   LevelExecutor& forward() {
     if (frozen_ && fused_ready_) {
       run_fused(kForward);
+      for (PendingInPlace* p : pending_steps_) p->settle();
       return *this;
     }
     if (frozen_) {
@@ -822,6 +835,7 @@ class LevelExecutor {
         }
         if (step.plan >= 0) launch(plans_[kForward][static_cast<size_t>(step.plan)]);
       }
+      for (PendingInPlace* p : pending_steps_) p->settle();
       return *this;
     }
     cursor_ = 0;
@@ -839,6 +853,7 @@ class LevelExecutor {
       }
       flush(kForward, step);
     }
+    for (PendingInPlace* p : pending_steps_) p->settle();
     return *this;
   }
 
@@ -859,7 +874,7 @@ class LevelExecutor {
     cursor_ = 0;
     descs_.clear();
     lazy_.clear();
-    const std::vector<unsigned char> lazy = lazy_grad_candidates(list_);
+    const std::vector<unsigned char> lazy = lazy_grad_candidates(list_, id_);
     Step& step = begin_step(kReset, 0);
     for (size_t i = 0; i < list_.size(); ++i) {  // graph order: views map onto gradients sized before them
       BaseNode* n = list_[i].get();
@@ -879,7 +894,7 @@ class LevelExecutor {
   // level; reset_grad() must have run (ginn/node.h:237-254).
   LevelExecutor& backward(double loss_coeff = 1) {
     seed_sink(loss_coeff);
-    internal::FoldWindow folds;  // row sums into leaf gradients are folded once, at the end
+    internal::FoldWindow folds(id_);  // row sums into leaf gradients are folded once, at the end
     if (frozen_) {
       if (fused_ready_) {
         run_fused(kBackward);

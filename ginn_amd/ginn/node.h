@@ -130,6 +130,9 @@ class BaseNode {
   // graphs that share nodes must not run at the same time.
   mutable uint64_t mark_epoch_ = 0;
   mutable size_t mark_value_ = 0;
+  // The pass (Graph / LevelExecutor id) in which this node is an input of
+  // exactly one node, i.e. in which its gradient has a single writer; 0 = none.
+  mutable uint64_t sole_user_pass_ = 0;
 
  public:
   bool forwarded = false;
@@ -144,6 +147,8 @@ class BaseNode {
     mark_value_ = value;
   }
   size_t mark_value() const { return mark_value_; }
+  uint64_t sole_user_pass() const { return sole_user_pass_; }
+  void set_sole_user_pass(uint64_t pass) const { sole_user_pass_ = pass; }
 
   BaseNode() = default;
   BaseNode(std::vector<BaseNodePtr> ins) : ins_(std::move(ins)) {}
@@ -330,13 +335,21 @@ class FoldWindow {
     thread_local std::vector<void (*)(int)> v;
     return v;
   }
+  static uint64_t& pass_id() {
+    thread_local uint64_t id = 0;
+    return id;
+  }
 
  public:
-  FoldWindow() { ++depth(); }
+  // `pass`: the id of the Graph / LevelExecutor whose backward pass this is (0: unknown).
+  explicit FoldWindow(uint64_t pass = 0) {
+    if (++depth() == 1) pass_id() = pass;
+  }
   FoldWindow(const FoldWindow&) = delete;
   FoldWindow& operator=(const FoldWindow&) = delete;
   ~FoldWindow() {
     if (--depth() != 0) return;
+    pass_id() = 0;
     if (!hooks().empty()) {  // left by an exception: nothing stays queued
       for (auto* fn : hooks()) fn(0);
       hooks().clear();
@@ -347,6 +360,8 @@ class FoldWindow {
     }
   }
   static bool open() { return depth() > 0; }
+  // The id of the outermost open pass on this thread; 0 when none or unknown.
+  static uint64_t pass() { return depth() > 0 ? pass_id() : 0; }
   static void note(ginn_hip_ctx* ctx) {
     auto& v = touched();
     if (std::find(v.begin(), v.end(), ctx) == v.end()) v.push_back(ctx);
@@ -385,9 +400,20 @@ class FoldWindow {
 // product's operands), the pass goes on without waiting for it, and the end of the pass waits for
 // the second stream.  The operands are a node's gradient and another node's value (or a buffer
 // the node keeps), none of which changes before the next pass.  Same kernels, same results.
+// The second stream is ordered behind what the pass had enqueued when the product was issued, not
+// against what the pass enqueues later: a leaf qualifies only when the running pass has exactly ONE
+// writer of its gradient (the leaf is an input of one node of the pass's graph, counted when the
+// graph's gradients were last reset: BaseNode::sole_user_pass()).  A weight that several nodes
+// share (tied weights, the cells of an unrolled recurrent net, a weight that is also summed by an
+// Add) keeps all of its gradient writers on the pass's own stream.
 inline bool& beside_pass_flag() {
   static bool on = true;
   return on;
+}
+// Launches sent to a second stream since the process began (for tests).
+inline std::atomic<size_t>& beside_launches() {
+  static std::atomic<size_t> n{0};
+  return n;
 }
 class BesidePass {
   static std::vector<std::pair<ginn_hip_ctx*, ginn_hip_ctx*>>& joined() {
@@ -411,6 +437,7 @@ class BesidePass {
     const size_t idx = dev->id().idx;
     ginn_hip_ctx* main = contexts().at(idx);
     if (!beside_pass_flag() || !FoldWindow::open() || !target.inputs().empty() || flops < kWorthIt) return main;
+    if (FoldWindow::pass() == 0 || target.sole_user_pass() != FoldWindow::pass()) return main;
     ginn_hip_ctx* beside = contexts().beside(idx);
     int ordered = 0;
     GINN_HIP_CALL(ginn_hip_ctx_wait_for(beside, main, &ordered));
@@ -418,6 +445,7 @@ class BesidePass {
     auto& v = joined();
     if (std::find(v.begin(), v.end(), std::make_pair(main, beside)) == v.end()) v.emplace_back(main, beside);
     FoldWindow::at_close(&join, /*first=*/true);
+    ++beside_launches();
     return beside;
   }
 };
@@ -464,10 +492,13 @@ inline bool lazy_grad_reset() { return internal::lazy_grad_reset_flag(); }
 // of list[i] may be flagged instead of zeroed.  That takes storage of its own,
 // exactly one use as an input within the list, and a user that overwrites --
 // directly, or through a chain of views and in-place nodes each with one use.
-inline std::vector<unsigned char> lazy_grad_candidates(const std::vector<BaseNodePtr>& list) {
+// With a pass id, every leaf of the list that is an input of exactly one node
+// is also noted as having a single gradient writer in that pass
+// (internal::BesidePass), and every other leaf as having several.
+inline std::vector<unsigned char> lazy_grad_candidates(const std::vector<BaseNodePtr>& list, uint64_t pass = 0) {
   const size_t n = list.size();
   std::vector<unsigned char> out(n, 0);
-  if (!internal::lazy_grad_reset_flag()) return out;
+  if (!internal::lazy_grad_reset_flag() && pass == 0) return out;
   const uint64_t epoch = BaseNode::new_epoch();
   for (size_t i = 0; i < n; ++i) list[i]->mark(epoch, i);
   std::vector<uint32_t> uses(n, 0), user(n, 0), slot(n, 0);
@@ -481,6 +512,10 @@ inline std::vector<unsigned char> lazy_grad_candidates(const std::vector<BaseNod
       slot[j] = static_cast<uint32_t>(k);
     }
   }
+  if (pass != 0)
+    for (size_t j = 0; j < n; ++j)
+      if (list[j]->inputs().empty()) list[j]->set_sole_user_pass(uses[j] == 1 ? pass : 0);
+  if (!internal::lazy_grad_reset_flag()) return out;
   std::vector<unsigned char> overwritten(n, 0);  // by the one user, were the gradient flagged
   for (size_t j = n; j-- > 0;) {                 // users come later in the list
     BaseNode& node = *list[j];
@@ -495,8 +530,32 @@ inline std::vector<unsigned char> lazy_grad_candidates(const std::vector<BaseNod
   return out;
 }
 
+// An in-place step (scale, mask) that postpones its work until somebody reads
+// its value: a Softmax directly after it then does scale, mask and softmax as
+// one launch over the scores (ginn_hip_scaled_masked_softmax_fwd) instead of
+// three.  Whoever else reads the value first triggers the step as usual.
+class PendingInPlace {
+ public:
+  enum class Step { Scale, Mask };
+  virtual ~PendingInPlace() = default;
+  virtual Step pending_step() const = 0;
+  virtual bool pending() const = 0;
+  virtual void take_pending() = 0;             // the caller does the step itself
+  virtual float pending_value() const = 0;     // the factor, or the value for masked entries
+  virtual BaseNode* pending_mask() const { return nullptr; }
+  virtual BaseNode* pending_input() const = 0;  // the node whose storage the step writes over
+  virtual void skip_next_backward() = 0;        // the caller has done this step's backward too
+  // Runs the step now if it is still pending.  Graph::forward() and
+  // LevelExecutor::forward() call this for every such node when the pass ends,
+  // so that the storage written over holds the final contents for any reader
+  // once forward() has returned (ginn/node/inplace.h:104-123, 152-212).
+  virtual void settle() = 0;
+};
+
 class Graph {
   std::vector<BaseNodePtr> list_;
+  std::vector<PendingInPlace*> pending_steps_;  // the nodes of list_ that may postpone their work
+  uint64_t id_ = BaseNode::new_epoch();  // names this graph's passes (copies hold the same list)
 
   // Depth-first, a node after all of its inputs, without recursion: the
   // depth of a graph is its longest path (a recurrent net unrolled over
@@ -526,10 +585,15 @@ class Graph {
     // A node is appended after all of its inputs; it is marked on entry,
     // which is equivalent for an acyclic graph.
     visit(sink, BaseNode::new_epoch());
+    for (auto& e : list_)
+      if (auto* p = dynamic_cast<PendingInPlace*>(e.get())) pending_steps_.push_back(p);
   }
 
+  // In-place steps that nobody has asked for by the end of the pass run then
+  // (PendingInPlace): after forward() every tensor holds its final contents.
   Graph& forward() {
     for (auto& e : list_) e->forward();
+    for (PendingInPlace* p : pending_steps_) p->settle();
     return *this;
   }
 
@@ -549,7 +613,7 @@ class Graph {
     } else {
       GINN_THROW("Unexpected scalar type in sink node!");
     }
-    internal::FoldWindow folds;
+    internal::FoldWindow folds(id_);
     for (auto it = list_.rbegin(); it != list_.rend(); ++it)
       if ((*it)->has_grad()) (*it)->backward();
     folds.close();
@@ -563,7 +627,7 @@ class Graph {
   // Gradients with a single overwriting user are flagged, not zeroed
   // (BaseNode::GradUse); all others are zeroed as in ginn/node.h:218-222.
   Graph& reset_grad() {
-    const std::vector<unsigned char> lazy = lazy_grad_candidates(list_);
+    const std::vector<unsigned char> lazy = lazy_grad_candidates(list_, id_);
     for (size_t i = 0; i < list_.size(); ++i) {
       if (lazy[i]) list_[i]->reset_grad_lazy();
       else list_[i]->reset_grad();

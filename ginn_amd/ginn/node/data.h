@@ -68,23 +68,6 @@ class BaseDataNode : public Node<Scalar> {
   std::string name() const override = 0;
 };
 
-// An in-place step (scale, mask) that postpones its work until somebody reads
-// its value: a Softmax directly after it then does scale, mask and softmax as
-// one launch over the scores (ginn_hip_scaled_masked_softmax_fwd) instead of
-// three.  Whoever else reads the value first triggers the step as usual.
-class PendingInPlace {
- public:
-  enum class Step { Scale, Mask };
-  virtual ~PendingInPlace() = default;
-  virtual Step pending_step() const = 0;
-  virtual bool pending() const = 0;
-  virtual void take_pending() = 0;             // the caller does the step itself
-  virtual float pending_value() const = 0;     // the factor, or the value for masked entries
-  virtual BaseNode* pending_mask() const { return nullptr; }
-  virtual BaseNode* pending_input() const = 0;  // the node whose storage the step writes over
-  virtual void skip_next_backward() = 0;        // the caller has done this step's backward too
-};
-
 // Inside a node whose gradient tensor is a view of the WHOLE gradient of the
 // node IN (its input 0): the flag of a lazily reset gradient lives in IN.
 #define GINN_GRAD_IS_VIEW_OF(IN)                                                               \
@@ -104,9 +87,13 @@ class PendingInPlace {
 // Inside a node whose grad() IS the gradient tensor of the node IN (its input 0):
 // IN sizes and clears it, this node has nothing to prepare.
 #define GINN_GRAD_IS_ALIAS_OF(IN)                                                              \
-  void init_grad() override {}                                                                 \
   void reset_grad() override {}                                                                \
   bool describe_reset_grad(std::vector<LaunchDesc>&) override { return true; }                 \
+  GINN_GRAD_IS_ALIAS_OF_BUT_FOR_RESET(IN)
+
+// The same without reset_grad() / describe_reset_grad(), for nodes that keep state of their own per pass.
+#define GINN_GRAD_IS_ALIAS_OF_BUT_FOR_RESET(IN)                                                \
+  void init_grad() override {}                                                                 \
   bool owns_grad() const override { return false; }                                            \
   bool take_lazy_zero() override { return IN->take_lazy_zero(); }                              \
   bool lazy_zero() const override { return IN->lazy_zero(); }                                  \

@@ -14,7 +14,9 @@
 namespace ginn {
 
 // x *= val in place; the gradient is scaled in place on the way back
-// (ginn/node/inplace.h:104-123).
+// (ginn/node/inplace.h:104-123).  The scaling is done when the value is first
+// read (a Softmax behind a mask step takes it over, node/nlnode.h), at the
+// latest when the forward pass of the Graph / LevelExecutor ends.
 template <typename Scalar>
 class InPlaceProdScalarNode : public BaseDataNode<Scalar>, public PendingInPlace {
   NodePtr<Scalar> in_;
@@ -30,6 +32,7 @@ class InPlaceProdScalarNode : public BaseDataNode<Scalar>, public PendingInPlace
   void forward_() override {
     internal::require_gpu(in_->dev(), "InPlaceProdScalar");
     pending_ = true;
+    skip_backward_ = false;
   }
   void backward_() override {
     if (skip_backward_) {
@@ -59,7 +62,12 @@ class InPlaceProdScalarNode : public BaseDataNode<Scalar>, public PendingInPlace
   float pending_value() const override { return val_; }
   BaseNode* pending_input() const override { return in_.get(); }
   void skip_next_backward() override { skip_backward_ = true; }
-  GINN_GRAD_IS_ALIAS_OF(in_)
+  void settle() override { (void)std::as_const(*this).value(); }
+  // A skip that the pass it was meant for did not consume (a backward pass cut short, nodes run by
+  // hand) must not reach the next one; the executors therefore call reset_grad() here in every pass.
+  void reset_grad() override { skip_backward_ = false; }
+  bool describe_reset_grad(std::vector<LaunchDesc>&) override { return false; }
+  GINN_GRAD_IS_ALIAS_OF_BUT_FOR_RESET(in_)
   template <typename Val>
   InPlaceProdScalarNode(const NodePtr<Scalar>& in, Val val)
       : BaseDataNode<Scalar>({in}), in_(in), val_(static_cast<float>(val)) {}
@@ -92,6 +100,7 @@ class InPlaceMaskNode : public BaseDataNode<Scalar>, public PendingInPlace {
     GINN_ASSERT(mask_->value().size() > 0);
     internal::require_gpu(in_->dev(), "InPlaceMask");
     pending_ = true;
+    skip_backward_ = false;
   }
   void backward_() override {
     if (skip_backward_) {
@@ -122,7 +131,12 @@ class InPlaceMaskNode : public BaseDataNode<Scalar>, public PendingInPlace {
   BaseNode* pending_mask() const override { return mask_.get(); }
   BaseNode* pending_input() const override { return in_.get(); }
   void skip_next_backward() override { skip_backward_ = true; }
-  GINN_GRAD_IS_ALIAS_OF(in_)
+  void settle() override { (void)std::as_const(*this).value(); }
+  // A skip that the pass it was meant for did not consume (a backward pass cut short, nodes run by
+  // hand) must not reach the next one; the executors therefore call reset_grad() here in every pass.
+  void reset_grad() override { skip_backward_ = false; }
+  bool describe_reset_grad(std::vector<LaunchDesc>&) override { return false; }
+  GINN_GRAD_IS_ALIAS_OF_BUT_FOR_RESET(in_)
   template <typename Val>
   InPlaceMaskNode(const NodePtr<Scalar>& in, const NodePtr<Scalar>& mask, Val mask_val)
       : BaseDataNode<Scalar>({in, mask}), in_(in), mask_(mask), mask_val_(static_cast<float>(mask_val)) {}

@@ -142,6 +142,14 @@ int ginn_hip_free(ginn_hip_ctx* ctx, void* ptr);
  * read it (bytes held for reuse, and blocks the pool knows, in use or held). */
 int ginn_hip_pool_configure(ginn_hip_ctx* ctx, int enabled, size_t limit_bytes);
 int ginn_hip_pool_trim(ginn_hip_ctx* ctx);
+/* The most device memory ONE product (ginn_hip_gemm, ginn_hip_affine_fwd) may take from
+ * ginn_hip_malloc for copies of operands whose leading dimensions or addresses rule out
+ * 16-byte accesses (default 2 GiB; 0: products never allocate).  cuBLAS takes such
+ * operands in place (ginn/prod.h:46-62); here a large product on them runs on padded
+ * copies when they fit the budget and the device has the room, and in place on the
+ * any-shape kernel otherwise -- a product never fails for want of that memory.  The
+ * blocks go back to the context's cache of released blocks after the call. */
+int ginn_hip_gemm_temp_budget(ginn_hip_ctx* ctx, size_t bytes);
 int ginn_hip_pool_stats(ginn_hip_ctx* ctx, size_t* cached_bytes, size_t* blocks);
 
 /* Device::copy, GPU<-CPU branch: asynchronous on the stream
@@ -829,6 +837,8 @@ typedef struct ginn_hip_graph ginn_hip_graph;
 int ginn_hip_capture_begin(ginn_hip_ctx* ctx);
 int ginn_hip_capture_end(ginn_hip_ctx* ctx, ginn_hip_graph** graph);
 int ginn_hip_graph_launch(ginn_hip_graph* graph);
+/* Kernel launches in the recording (what one replay runs on the device). */
+int ginn_hip_graph_kernel_count(ginn_hip_graph* graph, size_t* kernels);
 int ginn_hip_graph_destroy(ginn_hip_graph* graph);
 
 /* ------------------------------------------------------------------ */

@@ -158,6 +158,116 @@ int shim_lazy_graph(int dtype, int lazy, int mode, int passes, int hs, int nh, i
 // Products into weight gradients on the second stream of the GPU (on by default) or on the one stream.
 void shim_set_beside_pass(int on) { set_beside_pass(on != 0); }
 
+// A weight with several gradient writers in one pass: W [d x d] is the left operand of a product of
+// 2 d^3 flops (large enough for the second stream when d >= 800), of a narrow product W x2 (always on
+// the pass's stream) and an operand of an Add; V [d x d] has the large product as its only user.
+// Three passes; out_dw / out_dv: the gradients of W and V after the last one.  out_beside: launches
+// that went to the second stream.  mode: 0 = Graph, 1 = executor, 2 = frozen executor.
+int shim_shared_weight_graph(int mode, int d, const float* w, const float* v, const float* x1, const float* x2,
+                             float* out_loss, float* out_dw, float* out_dv, long* out_beside) {
+  try {
+    const Size n = d;
+    auto W = weight_of<Real>({n, n}, w);
+    auto V = weight_of<Real>({n, n}, v);
+    auto X1 = data_of<Real>({n, n}, x1, false);
+    auto X2 = data_of<Real>({n, 8}, x2, false);
+    NodePtr<Real> big = Prod(NodePtr<Real>(W), NodePtr<Real>(X1));      // dW += d(big) X1^T: 2 d^3 flops
+    NodePtr<Real> alone = Prod(NodePtr<Real>(V), NodePtr<Real>(big));   // V's only user; also 2 d^3 flops
+    NodePtr<Real> small = Prod(NodePtr<Real>(W), NodePtr<Real>(X2));    // dW += d(small) X2^T
+    NodePtr<Real> added = Add(NodePtr<Real>(W), NodePtr<Real>(Tanh(alone)));  // dW += d(added)
+    auto loss = Add(NodePtr<Real>(Sum(NodePtr<Real>(Tanh(added)))), NodePtr<Real>(Sum(NodePtr<Real>(Sigmoid(small)))));
+    Graph g(loss);
+    auto pass = [&](auto& runner) {
+      runner.reset_forwarded();
+      runner.forward();
+      runner.reset_grad();
+      runner.backward(1.);
+    };
+    const size_t before = internal::beside_launches();
+    if (mode == 0) {
+      for (int i = 0; i < 3; ++i) pass(g);
+    } else {
+      LevelExecutor ex(g);
+      pass(ex);
+      if (mode == 2) ex.freeze();
+      for (int i = 1; i < 3; ++i) pass(ex);
+    }
+    gpu()->synchronize();
+    if (out_beside) *out_beside = static_cast<long>(internal::beside_launches() - before);
+    read_back(loss->value(), out_loss);
+    read_back(W->grad(), out_dw);
+    read_back(V->grad(), out_dv);
+    return 0;
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return 2;
+  }
+}
+
+// In-place steps that postpone their work (InPlaceProdScalar, InPlaceMask; ginn/node/inplace.h:104-123,
+// 152-212 overwrite the input in forward()).  scores = A B [3 x 2], scaled by 0.5, entries with mask 0 set to -5.
+// which: 0 = the mask step is the sink: nobody reads its value; 1 = a Softmax behind it takes the steps over;
+// both: out = the SCORES node's own value after Graph::forward() (what a holder of the upstream node sees).
+// 2, 3 = the same two through LevelExecutor::forward().
+// 4 = a skip left over by a backward pass that was cut short: the Softmax's backward is run by hand on a
+// flagged gradient (it does the two steps' backward itself and tells them to skip theirs), the steps' own
+// backward never runs; the next pass, with flagging off, needs them.  out = d(scores) of that pass followed by
+// d(scores) of the same pass on a fresh graph (6 + 6 values).
+int shim_inplace_semantics(int which, const float* a, const float* b, const float* mask, float* out) {
+  try {
+    auto build = [&](bool softmax, NodePtr<Real>& scores, NodePtr<Real>& top) {
+      auto A = data_of<Real>({3, 4}, a, true);
+      auto B = data_of<Real>({4, 2}, b, true);
+      auto M = data_of<Real>({3, 2}, mask, false);
+      scores = Prod(NodePtr<Real>(A), NodePtr<Real>(B));
+      NodePtr<Real> x = InPlaceProdScalar(scores, 0.5);
+      x = InPlaceMask(x, NodePtr<Real>(M), -5.f);
+      top = softmax ? NodePtr<Real>(Softmax(x)) : x;
+    };
+    NodePtr<Real> scores, top;
+    if (which <= 3) {
+      build(which % 2 == 1, scores, top);
+      Graph g(top);
+      if (which < 2) {
+        g.forward();
+      } else {
+        LevelExecutor ex(g);
+        ex.forward();
+      }
+      read_back(scores->value(), out);
+      return 0;
+    }
+    if (which == 4) {
+      struct Restore {
+        bool was = lazy_grad_reset();
+        ~Restore() { set_lazy_grad_reset(was); }
+      } restore;
+      for (int fresh = 0; fresh < 2; ++fresh) {
+        build(true, scores, top);
+        NodePtr<Real> loss = Sum(NodePtr<Real>(CwiseProd(top, top)));
+        Graph g(loss);
+        g.forward();
+        if (!fresh) {
+          set_lazy_grad_reset(true);
+          g.reset_grad();               // flags d(scores): the Softmax is the chain's only user
+          top->grad().fill(1.f);
+          top->backward();              // fused backward; tells the two steps to skip theirs
+        }
+        set_lazy_grad_reset(false);
+        g.reset_grad();
+        g.backward(1.);
+        read_back(scores->grad(), out + 6 * fresh);
+      }
+      return 0;
+    }
+    g_error = "unknown case";
+    return 1;
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return 2;
+  }
+}
+
 // What everybody but the one overwriting user sees of a flagged gradient.
 // which: 0 = read between reset_grad() and backward(): zeros, not what the
 // last pass left; 1 = two graphs that share a node, reset one after the other

@@ -375,3 +375,39 @@ def test_odd_leading_dimensions_of_large_products(dev, dt, op_a, op_b, m, n, k, 
     dev.sync()
     err = float((C.double().transpose(1, 2) - want).norm() / want.norm())
     assert err <= 2 * _bound(dt), err
+
+
+@pytest.mark.parametrize("dt", [capi.F16, capi.F32])
+@pytest.mark.parametrize("budget", [0, 1 << 20, None])
+def test_products_on_copies_keep_within_the_budget_for_temporaries(dev, dt, budget):
+    """A product on operands with odd leading dimensions may take device memory for padded copies
+    (ginn_hip_gemm_temp_budget; cuBLAS computes in place, ginn/prod.h:46-62).  With a budget of 0, or one
+    the copies do not fit, it runs in place on the any-shape kernel instead: same result, nothing taken
+    from the context's pool; with the default budget the copies are made and returned to the pool."""
+    from ctypes import byref, c_size_t
+    from gpu_util import torch_dtype
+    torch = dev.torch
+    m, n, k = 1501, 1503, 1505
+    A, B, lda, ldb = _operands(dev, dt, 0, 0, m, n, k, 1, 77)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    C = torch.randn(1, n, m, generator=g, device="cuda").to(torch_dtype(dt))
+    want = _expected(A, B, 0, 0) + 0.5 * C.double().transpose(1, 2)
+
+    def blocks():
+        cached, count = c_size_t(0), c_size_t(0)
+        dev.lib.call("ginn_hip_pool_stats", dev.ctx, byref(cached), byref(count))
+        return count.value
+
+    dev.lib.call("ginn_hip_pool_trim", dev.ctx)
+    before = blocks()
+    try:
+        if budget is not None:
+            dev.lib.call("ginn_hip_gemm_temp_budget", dev.ctx, budget)
+        dev.gemm(dt, 0, 0, m, n, k, A.data_ptr(), lda, B.data_ptr(), ldb, 0.5, C.data_ptr(), m)
+        dev.sync()
+    finally:
+        dev.lib.call("ginn_hip_gemm_temp_budget", dev.ctx, 2 << 30)
+    took = blocks() - before
+    assert (took == 0) if budget is not None else (took >= 3), took
+    err = float((C.double().transpose(1, 2) - want).norm() / want.norm())
+    assert err <= 2 * _bound(dt), err

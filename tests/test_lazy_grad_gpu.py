@@ -140,3 +140,69 @@ def test_weight_gradients_beside_the_pass_are_the_same_bits(shim, dt, mode):
     for g, w in zip(got_grads, want_grads):
         assert np.abs(w).max() > 0
         np.testing.assert_array_equal(g, w)
+
+
+@pytest.mark.parametrize("mode", ["graph", "executor", "frozen"])
+def test_a_weight_with_several_gradient_writers_stays_on_the_pass_stream(shim, mode):
+    """A product goes to the second stream only when its target has one gradient writer in the pass
+    (internal::BesidePass): the second stream is not ordered against what the pass enqueues later.
+    W feeds a 2.1 GFLOP product, a narrow product and an Add, so all three writers of dW stay on the
+    pass's stream; V feeds one 2.1 GFLOP product, which goes beside.  Loss and both gradients are
+    bit-identical to the run on one stream."""
+    d = 1024
+    rng = np.random.default_rng(5)
+    w, v, x1 = (np.asfortranarray(rng.uniform(-1, 1, (d, d)).astype(np.float32) / math.sqrt(d)) for _ in range(3))
+    x2 = np.asfortranarray(rng.uniform(-1, 1, (d, 8)).astype(np.float32))
+
+    def once(beside):
+        dw = np.zeros((d, d), np.float32, order="F")
+        dv = np.zeros((d, d), np.float32, order="F")
+        loss = np.zeros(1, np.float32)
+        n = ctypes.c_long(-1)
+        shim.shim_set_beside_pass(beside)
+        rc = shim.shim_shared_weight_graph(MODES[mode], d, fptr(w), fptr(v), fptr(x1), fptr(x2), fptr(loss),
+                                           fptr(dw), fptr(dv), ctypes.byref(n))
+        assert rc == 0, shim.lazy_last_error().decode()
+        return loss[0], dw, dv, n.value
+
+    try:
+        want_loss, want_dw, want_dv, none = once(0)
+        got_loss, got_dw, got_dv, beside = once(1)
+    finally:
+        shim.shim_set_beside_pass(1)
+    assert none == 0
+    assert beside == 3  # dV of each of the three passes; never dW
+    assert np.abs(want_dw).max() > 0 and np.abs(want_dv).max() > 0
+    assert got_loss == want_loss
+    np.testing.assert_array_equal(got_dw, want_dw)
+    np.testing.assert_array_equal(got_dv, want_dv)
+
+
+@pytest.mark.parametrize("which", [0, 1, 2, 3])
+def test_in_place_steps_have_run_when_forward_returns(shim, which):
+    """InPlaceProdScalar / InPlaceMask overwrite their input in forward() in the reference
+    (ginn/node/inplace.h:104-123, 152-212).  Here they may wait for their first reader (a Softmax takes
+    them over); whoever holds the node they write over must still see the final contents once
+    Graph::forward() / LevelExecutor::forward() has returned, also when nobody read their value."""
+    rng = np.random.default_rng(which)
+    a = np.asfortranarray(rng.uniform(-1, 1, (3, 4)).astype(np.float32))
+    b = np.asfortranarray(rng.uniform(-1, 1, (4, 2)).astype(np.float32))
+    mask = np.asfortranarray(np.array([[1, 0], [1, 1], [0, 1]], np.float32))
+    out = np.zeros((3, 2), np.float32, order="F")
+    assert shim.shim_inplace_semantics(which, fptr(a), fptr(b), fptr(mask), fptr(out)) == 0, shim.lazy_last_error().decode()
+    want = np.where(mask != 0, np.float32(0.5) * (a.astype(np.float64) @ b).astype(np.float32), np.float32(-5))
+    np.testing.assert_allclose(out, want, rtol=1e-6, atol=1e-7)
+
+
+def test_a_skipped_backward_does_not_leak_into_the_next_pass(shim):
+    """A fused Softmax backward tells the in-place steps below to skip theirs; when their backward never
+    runs in that pass, the next pass (which needs them) gives what a fresh graph gives."""
+    rng = np.random.default_rng(9)
+    a = np.asfortranarray(rng.uniform(-1, 1, (3, 4)).astype(np.float32))
+    b = np.asfortranarray(rng.uniform(-1, 1, (4, 2)).astype(np.float32))
+    mask = np.asfortranarray(np.array([[1, 0], [1, 1], [0, 1]], np.float32))
+    out = np.zeros(12, np.float32)
+    assert shim.shim_inplace_semantics(4, fptr(a), fptr(b), fptr(mask), fptr(out)) == 0, shim.lazy_last_error().decode()
+    assert np.abs(out[6:]).max() > 0
+    assert (out[6:].reshape(3, 2, order="F")[mask == 0] == 0).all()  # masked entries pass no gradient
+    np.testing.assert_array_equal(out[:6], out[6:])
