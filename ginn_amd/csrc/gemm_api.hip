@@ -52,11 +52,6 @@ int launch_gemm_realigned(ginn_hip_ctx* ctx, const GemmArgs& a) {
   bool fix_a = bad(a.A, a.lda), fix_b = bad(a.B, a.ldb);
   bool fix_c = bad(a.C, a.ldc) || (a.pre && bad(a.pre, a.ldc));
   const bool fix_bias = a.bias && reinterpret_cast<uintptr_t>(a.bias) % 16 != 0;
-  // A large 16-bit product with ragged rows (or ragged columns that the tuned kernels cannot mask) takes the
-  // same way although its operands are aligned: zero-padded to whole tiles it runs on the tuned kernels alone,
-  // which beats the cut of launch_gemm_ragged (fp16 4000^3: 217-240 us cut, 4095 x 4097 x 4099 212 us on copies).
-  if (a.dtype != GINN_HIP_F32 && (a.m % 128 != 0 || (a.op_b == GINN_HIP_OP_T && a.n % 128 != 0)))
-    fix_a = fix_b = fix_c = true;
   if (!fix_a && !fix_b && !fix_c && !fix_bias) return kUnsupported;
   // From where the copies pay (measured, any-shape kernel alone -> on copies, us): fp32 1001 x 1003 x 1005
   // 115 -> 56, 515 x 2049 x 515 75 -> 47, but 801 x 803 x 805 54 -> 62; fp16 with one operand to copy

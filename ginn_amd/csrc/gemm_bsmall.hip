@@ -33,6 +33,7 @@ struct Params {
   long long sa, sb, sc;
   int tiles_m, tiles_n;  // per slice
   int batch;
+  int whole_lines;  // columns of C start on 128-byte lines
   int xcd_spread;  // workgroup ids are dealt to 8 XCDs round robin: give every XCD a contiguous run of slices
 };
 
@@ -48,7 +49,9 @@ struct GeoB {
   }
 };
 
-template <typename T, bool AKC, bool BKC, int FM, int FN>
+// EDGE: extents that are no multiples of the tile (or result columns that do not start on 128-byte
+// lines): masked stores through the cache; without it every store is a whole line and non-temporal.
+template <typename T, bool AKC, bool BKC, int FM, int FN, bool EDGE>
 __global__ __launch_bounds__(kThreadsB) void gemm_bsmall_kernel(Params p) {
   using G = GeoB<FM, FN>;
   constexpr int ES = 2;
@@ -68,7 +71,12 @@ __global__ __launch_bounds__(kThreadsB) void gemm_bsmall_kernel(Params p) {
   const long long bz = pid / tiles;
   const int tile = pid % tiles;
   const int m0 = (tile % p.tiles_m) * G::BM, n0 = (tile / p.tiles_m) * G::BN;
-  const int KT = p.k / BK;
+  const int KT = (p.k + BK - 1) / BK;
+  // K values in the last K tile (64 unless K is no multiple of the tile): the lanes whose 16 bytes of that
+  // tile lie beyond them load zeros.  Tile rows beyond m / n re-read rows inside the matrix (chunk_src) and
+  // what they produce is not stored.
+  const int k_lim = p.k - (KT - 1) * BK;
+  const int m_valid = EDGE ? min(G::BM, p.m - m0) : G::BM, n_valid = EDGE ? min(G::BN, p.n - n0) : G::BN;
 
   f32x16 acc[FM][FN];
 #pragma unroll
@@ -82,9 +90,16 @@ __global__ __launch_bounds__(kThreadsB) void gemm_bsmall_kernel(Params p) {
   constexpr int kPassA = 2 * FM, kPassB = 2 * FN;  // (64 F rows x 8 chunks) / 256 threads
   uint32_t a_off[kPassA], b_off[kPassB];
 #pragma unroll
-  for (int i = 0; i < kPassA; ++i) a_off[i] = (uint32_t)(chunk_src<AKC, FM, ES>(i * kThreadsB + tid, p.lda) * ES);
+  for (int i = 0; i < kPassA; ++i)
+    a_off[i] = (uint32_t)(chunk_src<AKC, FM, ES>(i * kThreadsB + tid, p.lda, m_valid) * ES);
 #pragma unroll
-  for (int i = 0; i < kPassB; ++i) b_off[i] = (uint32_t)(chunk_src<BKC, FN, ES>(i * kThreadsB + tid, p.ldb) * ES);
+  for (int i = 0; i < kPassB; ++i)
+    b_off[i] = (uint32_t)(chunk_src<BKC, FN, ES>(i * kThreadsB + tid, p.ldb, n_valid) * ES);
+  // This thread's chunk along K of a K-contiguous tile (the same in every pass); its k-row of pass 0 of a
+  // row-contiguous tile (8 FM or 8 FN chunks per k-row).
+  const bool kc_ok = (((tid & 7) ^ swz_kc(tid >> 3)) * 8) < k_lim;
+  constexpr int kRowsPerPassA = kThreadsB / (8 * FM), kRowsPerPassB = kThreadsB / (8 * FN);
+  const int a_rc_kr = tid / (8 * FM), b_rc_kr = tid / (8 * FN);
   const long long a_kstep = (AKC ? (long long)BK : (long long)BK * p.lda) * ES;
   const long long b_kstep = (BKC ? (long long)BK : (long long)BK * p.ldb) * ES;
   const char* a_next =
@@ -113,6 +128,29 @@ __global__ __launch_bounds__(kThreadsB) void gemm_bsmall_kernel(Params p) {
     }
     a_next += a_kstep;
     b_next += b_kstep;
+  };
+  // The last K tile: per-lane addresses, zeros beyond K.
+  auto issue_last_tile = [&](int buf) {
+    const char* zeros = reinterpret_cast<const char*>(kZeroChunk);
+#pragma unroll
+    for (int i = 0; i < kPassA; ++i) {
+      const bool ok = AKC ? kc_ok : (i * kRowsPerPassA + a_rc_kr) < k_lim;
+      const char* g = ok ? a_next + a_off[i] : zeros;
+      __builtin_amdgcn_global_load_lds(
+          (const void __attribute__((address_space(1)))*)g,
+          (void __attribute__((address_space(3)))*)(lds + buf * G::kStageBytes + (i * kThreadsB + wave * 64) * 16), 16,
+          0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < kPassB; ++i) {
+      const bool ok = BKC ? kc_ok : (i * kRowsPerPassB + b_rc_kr) < k_lim;
+      const char* g = ok ? b_next + b_off[i] : zeros;
+      __builtin_amdgcn_global_load_lds(
+          (const void __attribute__((address_space(1)))*)g,
+          (void __attribute__((address_space(3)))*)(lds + buf * G::kStageBytes + G::kTileA +
+                                                    (i * kThreadsB + wave * 64) * 16),
+          16, 0, 0);
+    }
   };
   constexpr int kLoads = kPassA + kPassB;
 
@@ -198,10 +236,14 @@ __global__ __launch_bounds__(kThreadsB) void gemm_bsmall_kernel(Params p) {
   };
 
   // ---- K loop: tile kt + 1 is on its way while tile kt is multiplied.
-  issue_tile(0);
+  const bool ragged_k = EDGE && k_lim != BK;
+  if (KT == 1 && ragged_k) issue_last_tile(0);
+  else issue_tile(0);
   for (int kt = 0; kt < KT; ++kt) {
     if (kt + 1 < KT) {
-      issue_tile((kt + 1) & 1);  // its stage was read last for tile kt - 1: every wave is past the barrier below
+      // its stage was read last for tile kt - 1: every wave is past the barrier below
+      if (kt + 2 == KT && ragged_k) issue_last_tile((kt + 1) & 1);
+      else issue_tile((kt + 1) & 1);
       asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kLoads) : "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -234,20 +276,35 @@ __global__ __launch_bounds__(kThreadsB) void gemm_bsmall_kernel(Params p) {
   for (int it = 0; it < 32 * FN / kColsPerIter; ++it) {
     const int col = it * kColsPerIter + sub;
     const u32x4 v = *reinterpret_cast<const u32x4*>(stage + col * G::kEpiColStride + chunk * 16);
-    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (long long)(n0 + wn + col) * p.ldc + m0 + wm + chunk * 8));
+    u32x4* dst = reinterpret_cast<u32x4*>(C + (long long)(n0 + wn + col) * p.ldc + m0 + wm + chunk * 8);
+    if constexpr (EDGE) {
+      // Neighbouring workgroups complete each other's 128-byte lines, which only the cache can merge
+      // (T = 504: 20.8 us with non-temporal stores, 13.1 us with these).
+      if (wn + col < n_valid && wm + chunk * 8 < m_valid) *dst = v;
+    } else {
+      __builtin_nontemporal_store(v, dst);
+    }
   }
 }
 
 template <typename T, bool AKC, bool BKC, int FM, int FN>
 int launch_one(ginn_hip_ctx* ctx, const Params& p) {
   using G = GeoB<FM, FN>;
-  const int stages = p.k / 64 > 1 ? 2 : 1;
+  const int stages = p.k > 64 ? 2 : 1;
   const int lds_bytes = G::lds_bytes(stages);
-  auto fn = gemm_bsmall_kernel<T, AKC, BKC, FM, FN>;
-  static std::atomic<unsigned long long> lds_allowed{0};
-  GH_HIP(allow_dynamic_lds(lds_allowed, ctx->device, reinterpret_cast<const void*>(fn), G::lds_bytes(2)));
   const long long blocks = (long long)p.tiles_m * p.tiles_n * p.batch;
-  fn<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreadsB), lds_bytes, ctx->stream>>>(p);
+  const bool edge = p.m % G::BM != 0 || p.n % G::BN != 0 || p.k % 64 != 0 || !p.whole_lines;
+  if (edge) {
+    auto fn = gemm_bsmall_kernel<T, AKC, BKC, FM, FN, true>;
+    static std::atomic<unsigned long long> lds_allowed{0};
+    GH_HIP(allow_dynamic_lds(lds_allowed, ctx->device, reinterpret_cast<const void*>(fn), G::lds_bytes(2)));
+    fn<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreadsB), lds_bytes, ctx->stream>>>(p);
+  } else {
+    auto fn = gemm_bsmall_kernel<T, AKC, BKC, FM, FN, false>;
+    static std::atomic<unsigned long long> lds_allowed{0};
+    GH_HIP(allow_dynamic_lds(lds_allowed, ctx->device, reinterpret_cast<const void*>(fn), G::lds_bytes(2)));
+    fn<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreadsB), lds_bytes, ctx->stream>>>(p);
+  }
   GH_HIP(hipGetLastError());
   return kOk;
 }
@@ -276,7 +333,12 @@ int launch_gemm_bsmall(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (a.dtype != GINN_HIP_F16 && a.dtype != GINN_HIP_BF16) return kUnsupported;
   if (a.batch < 2 || a.beta != 0.f || a.bias || a.pre || a.act != GINN_HIP_ACT_IDENTITY || a.bcols || a.ccols)
     return kUnsupported;
-  if (a.m % 64 || a.n % 64 || a.k % 64 || a.k < 64) return kUnsupported;
+  if (a.k < 64) return kUnsupported;
+  // Extents need not be multiples of the tile (a sequence length of 504): the last tile row / column and
+  // the last K tile are masked inside the kernel; every run of elements that is contiguous in memory must
+  // be a whole number of 16-byte chunks.
+  if (a.m % 8 || (a.op_b == GINN_HIP_OP_T && a.n % 8)) return kUnsupported;
+  if ((a.op_a == GINN_HIP_OP_T || a.op_b == GINN_HIP_OP_N) && a.k % 8) return kUnsupported;
   // Slices of little arithmetic per byte: one side of 64 (the head size) or a single K tile, and small enough
   // that a slice is a handful of tiles; the other batched shapes gain from the deeper pipeline of gemm_mid.h.
   const bool slim = a.k == 64 || a.m == 64 || a.n == 64;
@@ -285,7 +347,10 @@ int launch_gemm_bsmall(ginn_hip_ctx* ctx, const GemmArgs& a) {
   auto aligned16 = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
   if (!aligned16(a.A) || !aligned16(a.B) || !aligned16(a.C)) return kUnsupported;
   if ((long long)a.lda * 128 * 2 >= (1ll << 31) || (long long)a.ldb * 128 * 2 >= (1ll << 31)) return kUnsupported;
-  const int fm = a.m % 128 == 0 ? 2 : 1, fn = a.n % 128 == 0 ? 2 : 1;
+  // 128-wide tiles unless the extent is a multiple of 64 only, or a ragged one whose last 128 would be
+  // less than half full.
+  auto wide = [](int extent) { return extent % 128 == 0 || (extent % 64 != 0 && (extent - 1) % 128 >= 64) ? 2 : 1; };
+  const int fm = wide(a.m), fn = wide(a.n);
   bsmall::Params p;
   p.A = a.A;
   p.B = a.B;
@@ -299,9 +364,10 @@ int launch_gemm_bsmall(ginn_hip_ctx* ctx, const GemmArgs& a) {
   p.sa = a.stride_a;
   p.sb = a.stride_b;
   p.sc = a.stride_c;
-  p.tiles_m = a.m / (64 * fm);
-  p.tiles_n = a.n / (64 * fn);
+  p.tiles_m = (a.m + 64 * fm - 1) / (64 * fm);
+  p.tiles_n = (a.n + 64 * fn - 1) / (64 * fn);
   p.batch = a.batch;
+  p.whole_lines = a.ldc % 64 == 0 && a.stride_c % 64 == 0 && reinterpret_cast<uintptr_t>(a.C) % 128 == 0;
   const long long blocks = (long long)p.tiles_m * p.tiles_n * a.batch;
   if (blocks < ctx->num_cus || blocks > (1ll << 30)) return kUnsupported;
   p.xcd_spread = blocks % 8 == 0 ? 1 : 0;

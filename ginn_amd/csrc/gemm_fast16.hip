@@ -39,6 +39,10 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+// Sixteen zero bytes in device memory: where a direct load must deliver zeros (K values beyond the end of
+// a ragged K) its lane reads them from here instead of the operand.
+__device__ __attribute__((aligned(16))) const unsigned int kZeroChunk[4] = {0u, 0u, 0u, 0u};
+
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int kThreads = 256;
 constexpr int kTileBytes = 256 * BK * 2;       // one operand, one stage: 32 KiB
@@ -70,14 +74,19 @@ __device__ __forceinline__ int swz_rc(int kr) { return 4 * (kr & 3); }
 
 // Element offset, relative to the tile origin at K offset 0, of the 16-byte
 // chunk that lands at linear LDS chunk position v of the tile.
+// Tile rows from `valid` on (a tile that reaches beyond the matrix) re-read a
+// row inside it -- K-contiguous operand: the last valid row; row-contiguous
+// operand: the 16 bytes at the tile's first row (extents along the rows are
+// multiples of 8) -- in bounds, and what they produce is never stored.
 template <bool KC>
-__device__ __forceinline__ long long chunk_src(int v, int ld) {
+__device__ __forceinline__ long long chunk_src(int v, int ld, int valid) {
   if (KC) {
     const int row = v >> 3, pc = v & 7;
-    return (long long)row * ld + ((pc ^ swz_kc(row)) * 8);
+    return (long long)min(row, valid - 1) * ld + ((pc ^ swz_kc(row)) * 8);
   }
   const int kr = v >> 5, pj = v & 31;
-  return (long long)kr * ld + ((pj ^ swz_rc(kr)) * 8);
+  const int row0 = (pj ^ swz_rc(kr)) * 8;
+  return (long long)kr * ld + (row0 < valid ? row0 : 0);
 }
 
 // Byte offset inside a K-contiguous tile of lane's 16 bytes of the fragment
@@ -189,22 +198,29 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int KT = p.k / BK;
+  const int KT = (p.k + BK - 1) / BK;
+  // K values in the last K tile (64 unless K is no multiple of the tile): lanes
+  // whose 16 bytes of that tile lie beyond them load zeros instead.
+  const int k_lim = p.k - (KT - 1) * BK;
+  const int m_valid = min(BM, p.m - m0), n_valid = min(BN, p.n - n0);
 
   // Thread `tid` moves chunk v = i * 256 + tid (i = 0..7) of each operand; the
   // lane-dependent part of the source offset does not depend on i because the
   // swizzle only involves row bits below 32 (KC) / k bits below 8 (RC).  A
   // load takes a scalar tile origin plus a 32-bit per-thread offset.
-  const long long a_istep = (AKC ? 32ll * p.lda : 8ll * p.lda) * 2;
-  const long long b_istep = (BKC ? 32ll * p.ldb : 8ll * p.ldb) * 2;
   const long long a_kstep = (AKC ? (long long)BK : (long long)BK * p.lda) * 2;
   const long long b_kstep = (BKC ? (long long)BK : (long long)BK * p.ldb) * 2;
   uint32_t a_off[8], b_off[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    a_off[i] = (uint32_t)(chunk_src<AKC>(tid, p.lda) * 2 + i * a_istep);
-    b_off[i] = (uint32_t)(chunk_src<BKC>(tid, p.ldb) * 2 + i * b_istep);
+    a_off[i] = (uint32_t)(chunk_src<AKC>(i * kThreads + tid, p.lda, m_valid) * 2);
+    b_off[i] = (uint32_t)(chunk_src<BKC>(i * kThreads + tid, p.ldb, n_valid) * 2);
   }
+  // The chunk along K that this thread moves of a K-contiguous tile (the same in
+  // every pass) holds K values of the last tile; k-row of pass 0 of a
+  // row-contiguous tile (pass i: 8 i further).
+  const bool kc_ok = (((tid & 7) ^ swz_kc(tid >> 3)) * 8) < k_lim;
+  const int rc_kr = tid >> 5;
   const char* a_tile = reinterpret_cast<const char*>(p.A + bz * p.sa) +
                        (AKC ? (long long)m0 * p.lda : (long long)m0) * 2;
   const char* b_tile = reinterpret_cast<const char*>(p.B + bz * p.sb) +
@@ -219,6 +235,21 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
     uint32_t& off = (q & 1) ? b_off[i] : a_off[i];
     asm volatile("" : "+v"(off));  // keeps (scalar origin) + (32-bit offset) apart for the addressing mode
     const char* g = ((q & 1) ? gb : ga) + off;
+    const int vbase = i * kThreads + wave * 64;
+    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)g,
+                                     (void __attribute__((address_space(3)))*)(l + vbase * 16), 16,
+                                     0, 0);
+  };
+
+  // The same for the last K tile, which K may fill only in part: a per-lane
+  // address, the lanes beyond K read zeros.
+  auto issue_q_last = [&](const char* ga, const char* gb, int buf, int q) {
+    const int i = q >> 1;
+    char* l = lds + buf * kStageBytes + ((q & 1) ? kTileBytes : 0);
+    const bool kc = (q & 1) ? BKC : AKC;
+    const bool ok = kc ? kc_ok : (8 * i + rc_kr) < k_lim;
+    const char* g = ((q & 1) ? gb : ga) + ((q & 1) ? b_off[i] : a_off[i]);
+    if (!ok) g = reinterpret_cast<const char*>(kZeroChunk);
     const int vbase = i * kThreads + wave * 64;
     __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)g,
                                      (void __attribute__((address_space(3)))*)(l + vbase * 16), 16,
@@ -291,15 +322,21 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
   // One sub-step in pinned order: 16 MFMAs on fragment set f; between them the
   // 8 fragment reads of sub-step KS of the current stage (RD) and 8 direct
   // loads of the tile at ga / gb (LD), the latter after every other MFMA.
-  auto substep = [&](int f, auto rd_c, auto KS, auto ld_c, const char* ga, const char* gb, int lbuf, int lq0) {
+  // LAST: the tile loaded is the last one (loads by per-lane address).
+  auto substep = [&](int f, auto rd_c, auto KS, auto ld_c, auto last_c, const char* ga, const char* gb, int lbuf,
+                     int lq0) {
     constexpr bool RD = decltype(rd_c)::value;
     constexpr bool LD = decltype(ld_c)::value;
+    constexpr bool LAST = decltype(last_c)::value;
     static_for<16>([&](auto IDX) {
       constexpr int idx = decltype(IDX)::value;
       constexpr int i = idx >> 2, j = idx & 3;
       acc[i][j] = mma<BF>(__builtin_bit_cast(u16x8, qa[f][i]), __builtin_bit_cast(u16x8, qb[f][j]), acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (LD && (idx & 1) == 0) issue_q(ga, gb, lbuf, (idx >> 1) + lq0);
+      if constexpr (LD && (idx & 1) == 0) {
+        if constexpr (LAST) issue_q_last(ga, gb, lbuf, (idx >> 1) + lq0);
+        else issue_q(ga, gb, lbuf, (idx >> 1) + lq0);
+      }
       // B fragments first: the next sub-step's first four MFMAs need all of them.
       if constexpr (RD && idx < 8) read_one(KS, f ^ 1, std::integral_constant<int, (idx < 4 ? idx + 4 : idx - 4)>{});
       __builtin_amdgcn_sched_barrier(0);
@@ -320,7 +357,8 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
   // issued (first sub-step); NEXT: tile kt+1 exists; TAIL: tile kt+2 exists
   // (first half of its loads goes into the stage released by the barrier).
   // Compile-time flags keep every sub-step one basic block.
-  auto kstep = [&](int kt, auto head_c, auto next_c, auto tail_c) {
+  // HLAST / TLAST: the tile that HEAD / TAIL loads is the product's last one.
+  auto kstep = [&](int kt, auto head_c, auto next_c, auto tail_c, auto hlast_c, auto tlast_c) {
     constexpr bool HEAD = decltype(head_c)::value;
     constexpr bool NEXT = decltype(next_c)::value;
     constexpr bool TAIL = decltype(tail_c)::value;
@@ -330,9 +368,9 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
     const char* a_n2 = a_nx + a_kstep;
     const char* b_n2 = b_nx + b_kstep;
     asm volatile("" : "+s"(a_nx), "+s"(b_nx), "+s"(a_n2), "+s"(b_n2));
-    substep(0, std::true_type{}, K1, std::integral_constant<bool, HEAD>{}, a_nx, b_nx, buf ^ 1, 8);
-    substep(1, std::true_type{}, K2, std::false_type{}, nullptr, nullptr, 0, 0);
-    substep(0, std::true_type{}, K3, std::false_type{}, nullptr, nullptr, 0, 0);
+    substep(0, std::true_type{}, K1, std::integral_constant<bool, HEAD>{}, hlast_c, a_nx, b_nx, buf ^ 1, 8);
+    substep(1, std::true_type{}, K2, std::false_type{}, std::false_type{}, nullptr, nullptr, 0, 0);
+    substep(0, std::true_type{}, K3, std::false_type{}, std::false_type{}, nullptr, nullptr, 0, 0);
     // Every fragment read of tile kt has completed (finish); tile kt+1 must
     // have landed before anyone reads it, and the stage of tile kt is free
     // once all waves are here.
@@ -341,17 +379,26 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     if (NEXT) switch_stage(buf ? -kStageBytes : kStageBytes);
-    substep(1, std::integral_constant<bool, NEXT>{}, K0, std::integral_constant<bool, TAIL>{}, a_n2, b_n2, buf, 0);
+    substep(1, std::integral_constant<bool, NEXT>{}, K0, std::integral_constant<bool, TAIL>{}, tlast_c, a_n2, b_n2, buf,
+            0);
     a_nx = a_n2;
     b_nx = b_n2;
   };
 
   // Prologue: tiles 0 and 1 in full, first fragments of tile 0.
+  if (KT == 1) {
 #pragma unroll
-  for (int q = 0; q < 16; ++q) issue_q(a_tile, b_tile, 0, q);
-  if (KT > 1) {
+    for (int q = 0; q < 16; ++q) issue_q_last(a_tile, b_tile, 0, q);
+  } else {
 #pragma unroll
-    for (int q = 0; q < 16; ++q) issue_q(a_nx, b_nx, 1, q);
+    for (int q = 0; q < 16; ++q) issue_q(a_tile, b_tile, 0, q);
+    if (KT == 2) {
+#pragma unroll
+      for (int q = 0; q < 16; ++q) issue_q_last(a_nx, b_nx, 1, q);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 16; ++q) issue_q(a_nx, b_nx, 1, q);
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
@@ -361,17 +408,24 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
 
   using Y = std::true_type;
   using N = std::false_type;
+  // Tile t is loaded by the TAIL of K-step t - 2 and the HEAD of K-step t - 1:
+  // the last tile by K-steps KT - 3 and KT - 2, which are peeled for it.
   if (KT == 1) {
-    kstep(0, N{}, N{}, N{});
+    kstep(0, N{}, N{}, N{}, N{}, N{});
   } else if (KT == 2) {
-    kstep(0, N{}, Y{}, N{});
-    kstep(1, N{}, N{}, N{});
+    kstep(0, N{}, Y{}, N{}, N{}, N{});
+    kstep(1, N{}, N{}, N{}, N{}, N{});
   } else {
-    kstep(0, N{}, Y{}, Y{});
     int kt = 1;
-    for (; kt + 2 < KT; ++kt) kstep(kt, Y{}, Y{}, Y{});
-    kstep(kt, Y{}, Y{}, N{});
-    kstep(kt + 1, N{}, N{}, N{});
+    if (KT == 3) {
+      kstep(0, N{}, Y{}, Y{}, N{}, Y{});
+    } else {
+      kstep(0, N{}, Y{}, Y{}, N{}, N{});
+      for (; kt + 3 < KT; ++kt) kstep(kt, Y{}, Y{}, Y{}, N{}, N{});
+      kstep(kt++, Y{}, Y{}, Y{}, N{}, Y{});
+    }
+    kstep(kt, Y{}, Y{}, N{}, Y{}, N{});
+    kstep(kt + 1, N{}, N{}, N{}, N{}, N{});
   }
 
   // ------------------------------------------------------------------ epilogue
@@ -402,7 +456,8 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
     for (int it = 0; it < 32; ++it) {
       const int col = it * 4 + sub;
       const u32x4 v = *reinterpret_cast<const u32x4*>(stage + col * kEpiColStride + chunk * 16);
-      *reinterpret_cast<u32x4*>(C + (long long)(n0 + wn + col) * p.ldc + m0 + wm + chunk * 8) = v;
+      if (wn + col < n_valid && wm + chunk * 8 < m_valid)
+        *reinterpret_cast<u32x4*>(C + (long long)(n0 + wn + col) * p.ldc + m0 + wm + chunk * 8) = v;
     }
   } else {
     // General epilogue: C = act(acc + beta * C + bias), optionally keeping the
@@ -431,10 +486,11 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
     };
     auto read_pass = [&](int pass) {
       const int row = m0 + wm + chunk * 8;
+      const bool row_ok = wm + chunk * 8 < m_valid;  // m is a multiple of 8: a chunk of rows is inside or outside
       float bias8[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) bias8[e] = 0.f;
-      if (p.bias) {
+      if (p.bias && row_ok) {
         const u16x8 bv = *reinterpret_cast<const u16x8*>(p.bias + row);
 #pragma unroll
         for (int e = 0; e < 8; ++e) bias8[e] = to_float<T>(bv[e]);
@@ -443,6 +499,7 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
       const uint16_t* Cin = P ? P : C;
       // One column of the pass: 8 rows per lane from the staged fp32 tile.
       auto finish = [&](int lcol, bool with_old, const u16x8& old) {
+        if (!row_ok || wn + pass * 64 + lcol >= n_valid) return;
         const char* src = stage + lcol * kF32ColStride + chunk * 32;
         const f32x4 lo = *reinterpret_cast<const f32x4*>(src);
         const f32x4 hi = *reinterpret_cast<const f32x4*>(src + 16);
@@ -477,7 +534,9 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
 #pragma unroll
           for (int u = 0; u < kBatch; ++u) {
             const int lcol = (it0 + u) * 4 + sub;  // column inside the pass
-            old[u] = *reinterpret_cast<const u16x8*>(Cin + (long long)(n0 + wn + pass * 64 + lcol) * p.ldc + row);
+            old[u] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (row_ok && wn + pass * 64 + lcol < n_valid)
+              old[u] = *reinterpret_cast<const u16x8*>(Cin + (long long)(n0 + wn + pass * 64 + lcol) * p.ldc + row);
           }
 #pragma unroll
           for (int u = 0; u < kBatch; ++u) finish((it0 + u) * 4 + sub, true, old[u]);
@@ -528,14 +587,23 @@ int launch_layout(ginn_hip_ctx* ctx, const FastParams& p, int batch, bool akc, b
 int launch_gemm_fast16(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (a.dtype != GINN_HIP_F16 && a.dtype != GINN_HIP_BF16) return kUnsupported;
   if (a.bcols || a.ccols) return kUnsupported;
-  if (a.m % BM || a.n % BN || a.k % BK || a.k < 4 * BK) return kUnsupported;
+  if (a.k < 4 * BK) return kUnsupported;
+  // Extents need not be multiples of the tile: the last tile row / column and the last K tile are masked
+  // inside the kernel.  Every run of elements that is contiguous in memory (the rows of C and of a
+  // row-contiguous operand, K along a K-contiguous one) must be a whole number of 16-byte chunks.
+  if (a.m % 8 || (a.op_b == GINN_HIP_OP_T && a.n % 8)) return kUnsupported;
+  if ((a.op_a == GINN_HIP_OP_T || a.op_b == GINN_HIP_OP_N) && a.k % 8) return kUnsupported;
   if (a.lda % 8 || a.ldb % 8 || a.ldc % 8) return kUnsupported;
   auto aligned16 = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
   if (!aligned16(a.A) || !aligned16(a.B) || !aligned16(a.C)) return kUnsupported;
   if (a.pre && !aligned16(a.pre)) return kUnsupported;
   if (a.bias && reinterpret_cast<uintptr_t>(a.bias) % 8) return kUnsupported;
   if (a.batch > 1 && (a.stride_a % 8 || a.stride_b % 8 || a.stride_c % 8)) return kUnsupported;
-  const long long tiles = (long long)(a.m / BM) * (a.n / BN);
+  const int tiles_m = (a.m + BM - 1) / BM, tiles_n = (a.n + BN - 1) / BN;
+  const long long tiles = (long long)tiles_m * tiles_n;
+  // Tiles that reach beyond the matrix multiply for nothing: with more than an eighth of the work wasted
+  // the 128 x 128 kernel, whose edge tiles waste less, takes the product.
+  if ((double)tiles * BM * BN > 1.125 * (double)a.m * a.n) return kUnsupported;
   // With tiles for fewer than 9/16 of the CUs too much of the chip idles and
   // the 128 x 128 kernel is the better fit (measured, bf16: 3072^3 = 144 tiles
   // 61 us here against 78-79 us there; 2048 x 4096 x 2048 = 128 tiles level at
@@ -562,8 +630,8 @@ int launch_gemm_fast16(ginn_hip_ctx* ctx, const GemmArgs& a) {
   p.bias = static_cast<const uint16_t*>(a.bias);
   p.pre = static_cast<uint16_t*>(a.pre);
   p.act = a.act;
-  p.tiles_m = a.m / BM;
-  p.tiles_n = a.n / BN;
+  p.tiles_m = tiles_m;
+  p.tiles_n = tiles_n;
   const bool akc = a.op_a == GINN_HIP_OP_T;
   const bool bkc = a.op_b == GINN_HIP_OP_N;
   // XCD-aware ordering needs the tile count to split evenly over the 8 XCDs.

@@ -46,6 +46,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+// Sixteen zero bytes in device memory: where a direct load must deliver zeros (K values beyond the end of
+// a ragged K) its lane reads them from here instead of the operand.
+static __device__ __attribute__((aligned(16))) const unsigned int kZeroChunk[4] = {0u, 0u, 0u, 0u};
+
 constexpr int kRowBytes = 128;  // bytes of one K tile along K: 64 16-bit or 32 fp32 values
 constexpr int kThreads = 512;   // 8 waves
 constexpr int kStages = 4;
@@ -99,16 +103,19 @@ __device__ __forceinline__ int swz_rc(int kr) {
 // Element offset, relative to the tile origin at K offset 0, of the 16-byte
 // chunk that lands at linear LDS chunk position v of an operand tile of 64 F
 // rows; ES = element size in bytes.
+// Tile rows from `valid` on (a tile that reaches beyond the matrix) re-read a
+// row inside it: in bounds, and what they produce is never stored.
 template <bool KC, int F, int ES>
-__device__ __forceinline__ long long chunk_src(int v, int ld) {
+__device__ __forceinline__ long long chunk_src(int v, int ld, int valid) {
   constexpr int kPer = 16 / ES;  // elements per chunk
   if (KC) {
     const int row = v >> 3, pc = v & 7;
-    return (long long)row * ld + ((pc ^ swz_kc(row)) * kPer);
+    return (long long)min(row, valid - 1) * ld + ((pc ^ swz_kc(row)) * kPer);
   }
   constexpr int kChunks = 64 * F * ES / 16;  // per k-row
   const int kr = v / kChunks, pj = v % kChunks;
-  return (long long)kr * ld + ((pj ^ swz_rc<F, ES>(kr)) * kPer);
+  const int row0 = (pj ^ swz_rc<F, ES>(kr)) * kPer;  // first of the chunk's rows
+  return (long long)kr * ld + (row0 < valid ? row0 : 0);
 }
 
 // Byte offset inside a K-contiguous tile of lane's 16 bytes of the fragment
@@ -247,9 +254,12 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int kt_total = p.k / (kRowBytes / static_cast<int>(sizeof(typename T::storage)));
+  const int kt_total = (p.k + BK - 1) / BK;
   const int kt0 = split * p.k_tiles;
   const int KT = min(p.k_tiles, kt_total - kt0);
+  // K values in the last K tile of the product when K is no multiple of the tile (0: it is): the lanes
+  // whose 16 bytes lie beyond them load zeros instead.  Only the split that holds that tile sees it.
+  const int k_rem = (kt0 + KT == kt_total) ? p.k % BK : 0;
 
   // ---- direct loads.  Thread `tid` moves chunk v = i * 512 + tid (i < F) of an
   // operand tile; the swizzle only involves row bits below 32 (KC) / k bits
@@ -263,22 +273,38 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
   const long long b_istep = (BKC ? (long long)kRowsPerPass : (long long)kRcRowsPerPassB) * p.ldb * ES;
   const long long a_kstep = (AKC ? (long long)BK : (long long)BK * p.lda) * ES;
   const long long b_kstep = (BKC ? (long long)BK : (long long)BK * p.ldb) * ES;
-  // n need not fill the last tile column when B is K-contiguous (its tile rows
-  // are columns of the product): rows beyond n re-read the last valid one --
-  // in bounds, and what they produce is never stored.
-  const int n_valid = min(G::BN, p.n - n0);
+  // m and n need not fill the last tile row / column: tile rows beyond them
+  // re-read a valid one (K-contiguous operand: the last valid row; row-contiguous
+  // operand: the chunk of 16 bytes at the tile's first row, extents along the
+  // rows being multiples of 16 bytes) -- in bounds, and what they produce is
+  // never stored.
+  const int m_valid = min(G::BM, p.m - m0), n_valid = min(G::BN, p.n - n0);
   uint32_t a_off[FM], b_off[FN];  // byte offsets of this thread's chunks from the tile origin
 #pragma unroll
-  for (int i = 0; i < FM; ++i) a_off[i] = (uint32_t)(chunk_src<AKC, FM, ES>(tid, p.lda) * ES + i * a_istep);
+  for (int i = 0; i < FM; ++i) {
+    if (AKC) {
+      const int row = i * kRowsPerPass + (tid >> 3);
+      a_off[i] = (uint32_t)((long long)min(row, m_valid - 1) * p.lda * ES + (((tid & 7) ^ swz_kc(row)) * 16));
+    } else {
+      a_off[i] = (uint32_t)(chunk_src<AKC, FM, ES>(tid, p.lda, m_valid) * ES + i * a_istep);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < FN; ++i) {
     if (BKC) {
       const int row = i * kRowsPerPass + (tid >> 3);
       b_off[i] = (uint32_t)((long long)min(row, n_valid - 1) * p.ldb * ES + (((tid & 7) ^ swz_kc(row)) * 16));
     } else {
-      b_off[i] = (uint32_t)(chunk_src<BKC, FN, ES>(tid, p.ldb) * ES + i * b_istep);
+      b_off[i] = (uint32_t)(chunk_src<BKC, FN, ES>(tid, p.ldb, n_valid) * ES + i * b_istep);
     }
   }
+  // Whether this thread's chunk of the LAST, partly filled K tile holds K values
+  // of the product (K-contiguous operand: its chunk along K, the same in every
+  // pass; row-contiguous operand: the k-row, by pass).
+  constexpr int kPerChunk = 16 / ES;
+  const bool a_kc_ok = (((tid & 7) ^ swz_kc(tid >> 3)) * kPerChunk) < k_rem;
+  const bool b_kc_ok = a_kc_ok;
+  const int a_rc_kr = tid / (64 * FM * ES / 16), b_rc_kr = tid / (64 * FN * ES / 16);
   // Origins of the next tile to load (uniform).
   const char* a_next = static_cast<const char*>(p.A) +
                        (bz * p.sa + (AKC ? (long long)m0 * p.lda : (long long)m0)) * ES + kt0 * a_kstep;
@@ -308,6 +334,30 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
     }
     a_next += a_kstep;
     b_next += b_kstep;
+  };
+  // The same for the partly filled last K tile: a lane whose 16 bytes lie beyond
+  // K reads zeros (a per-lane address instead of scalar base + lane offset).
+  auto issue_last_tile = [&](int buf) {
+    const char* zeros = reinterpret_cast<const char*>(kZeroChunk);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      const bool ok = AKC ? a_kc_ok : (i * kRcRowsPerPassA + a_rc_kr) < k_rem;
+      const char* g = ok ? a_next + a_off[i] : zeros;
+      __builtin_amdgcn_global_load_lds(
+          (const void __attribute__((address_space(1)))*)g,
+          (void __attribute__((address_space(3)))*)(lds + buf * G::kStageBytes + (i * kThreads + wave * 64) * 16), 16, 0,
+          0);
+    }
+#pragma unroll
+    for (int i = 0; i < FN; ++i) {
+      const bool ok = BKC ? b_kc_ok : (i * kRcRowsPerPassB + b_rc_kr) < k_rem;
+      const char* g = ok ? b_next + b_off[i] : zeros;
+      __builtin_amdgcn_global_load_lds(
+          (const void __attribute__((address_space(1)))*)g,
+          (void __attribute__((address_space(3)))*)(lds + buf * G::kStageBytes + G::kTileA +
+                                                    (i * kThreads + wave * 64) * 16),
+          16, 0, 0);
+    }
   };
   constexpr int kLoads = FM + FN;  // direct loads per thread and K tile
   // Waits until at most `newer` whole tiles of this thread's direct loads are pending.
@@ -431,9 +481,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
   const std::integral_constant<int, 0> J0;
   const std::integral_constant<int, 1> J1;
 
-  // One K tile.  MORE: another tile follows; T2, T3: tiles kt + 2, kt + 3 exist.
-  auto k_tile = [&](int kt, auto MORE, auto T2, auto T3) {
+  // One K tile.  MORE: another tile follows; T2, T3: tiles kt + 2, kt + 3 exist;
+  // LAST: tile kt + 3 is the last one and may be partly filled.
+  auto k_tile = [&](int kt, auto MORE, auto T2, auto T3, auto LAST) {
     constexpr bool more = decltype(MORE)::value, t2 = decltype(T2)::value, t3 = decltype(T3)::value;
+    constexpr bool last = decltype(LAST)::value;
     __builtin_amdgcn_sched_barrier(0);
     if (more) {
       // Tile kt + 1 is needed from here on (the refills below read it): its
@@ -442,7 +494,10 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
       // reading tile kt - 1, whose stage the loads of tile kt + 3 overwrite.
       wait_tiles(t2 ? 1 : 0);
       __builtin_amdgcn_s_barrier();
-      if (t3) issue_tile((kt + kStages - 1) % kStages);
+      if (t3) {
+        if (last && k_rem != 0) issue_last_tile((kt + kStages - 1) % kStages);
+        else issue_tile((kt + kStages - 1) % kStages);
+      }
       set_stage((kt + 1) % kStages);
     }
     // A set is complete once only the reads of the other one are pending.
@@ -467,7 +522,10 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
   // Tiles 0 .. 2 go out at once; tile kt + 3 follows at the barrier of K tile kt.
 #pragma unroll
   for (int s = 0; s < kStages - 1; ++s)
-    if (s < KT) issue_tile(s);
+    if (s < KT) {
+      if (s == KT - 1 && k_rem != 0) issue_last_tile(s);
+      else issue_tile(s);
+    }
   wait_tiles(min(kStages - 2, KT - 1));
   __builtin_amdgcn_s_barrier();  // every wave's share of tile 0 is in LDS
   set_stage(0);
@@ -477,10 +535,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
     const std::true_type yes;
     const std::false_type no;
     int kt = 0;
-    for (; kt + 3 < KT; ++kt) k_tile(kt, yes, yes, yes);
-    if (kt + 2 < KT) k_tile(kt++, yes, yes, no);
-    if (kt + 1 < KT) k_tile(kt++, yes, no, no);
-    k_tile(kt, no, no, no);
+    for (; kt + 4 < KT; ++kt) k_tile(kt, yes, yes, yes, no);
+    if (kt + 3 < KT) k_tile(kt++, yes, yes, yes, yes);
+    if (kt + 2 < KT) k_tile(kt++, yes, yes, no, no);
+    if (kt + 1 < KT) k_tile(kt++, yes, no, no, no);
+    k_tile(kt, no, no, no, no);
   }
 
   {
@@ -524,7 +583,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
           const f32x4 v = {acc[i][j][4 * b], acc[i][j][4 * b + 1], acc[i][j][4 * b + 2], acc[i][j][4 * b + 3]};
           const size_t col = n0 + wn + j * 32 + l32;
           const size_t row = m0 + wm + i * 32 + 8 * b + 4 * lhi;
-          if (col < (size_t)p.n) *reinterpret_cast<f32x4*>(out + col * p.m + row) = v;
+          if (col < (size_t)p.n && row < (size_t)p.m) *reinterpret_cast<f32x4*>(out + col * p.m + row) = v;
         }
     return;
   }
@@ -544,7 +603,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
           f32x4 v = {acc[i][j][4 * b], acc[i][j][4 * b + 1], acc[i][j][4 * b + 2], acc[i][j][4 * b + 3]};
           const size_t col = n0 + wn + j * 32 + l32;
           const size_t row = m0 + wm + i * 32 + 8 * b + 4 * lhi;
-          if (col >= (size_t)p.n) continue;
+          if (col >= (size_t)p.n || row >= (size_t)p.m) continue;
           const size_t off = col * p.ldc + row;
           if (EPI == kGeneral) {
             if (p.beta != 0.f) v += p.beta * *reinterpret_cast<const f32x4*>((P ? P : C) + off);
@@ -586,7 +645,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
     for (int it = 0; it < 32 * FN / kColsPerIter; ++it) {
       const int col = it * kColsPerIter + sub;
       const u32x4 v = *reinterpret_cast<const u32x4*>(stage + col * G::kEpiColStride + chunk * 16);
-      if (n0 + wn + col < p.n)
+      if (n0 + wn + col < p.n && m0 + wm + chunk * 8 < p.m)
         *reinterpret_cast<u32x4*>(C + (long long)(n0 + wn + col) * p.ldc + m0 + wm + chunk * 8) = v;
     }
   } else {
@@ -595,10 +654,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
     // rounded once.
     uint16_t* P = p.pre ? static_cast<uint16_t*>(p.pre) + bz * p.sc : nullptr;
     const int row = m0 + wm + chunk * 8;
+    const bool row_ok = row < p.m;  // m is a multiple of 8: a chunk of rows is inside or outside
     float bias8[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) bias8[e] = 0.f;
-    if (p.bias) {
+    if (p.bias && row_ok) {
       const u16x8 bv = *reinterpret_cast<const u16x8*>(static_cast<const uint16_t*>(p.bias) + row);
 #pragma unroll
       for (int e = 0; e < 8; ++e) bias8[e] = to_float<T>(bv[e]);
@@ -623,7 +683,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
         for (int it = 0; it < kIters; ++it) {
           const int col = n0 + wn + pass * 32 + it * kColsPerIter + sub;
           old[it] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
-          if (col < p.n) old[it] = *reinterpret_cast<const u16x8*>(Cin + (long long)col * p.ldc + row);
+          if (col < p.n && row_ok) old[it] = *reinterpret_cast<const u16x8*>(Cin + (long long)col * p.ldc + row);
         }
       }
       GH_SWITCH_ACT(p.act, {
@@ -633,7 +693,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
           const f32x4 lo = *reinterpret_cast<const f32x4*>(src);
           const f32x4 hi = *reinterpret_cast<const f32x4*>(src + 16);
           float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          if (n0 + wn + pass * 32 + lcol < p.n) {
+          if (n0 + wn + pass * 32 + lcol < p.n && row_ok) {
             const long long off = (long long)(n0 + wn + pass * 32 + lcol) * p.ldc + row;
             if (p.beta != 0.f) {
               _Pragma("unroll") for (int e = 0; e < 8; ++e) v[e] += p.beta * to_float<T>(old[it][e]);

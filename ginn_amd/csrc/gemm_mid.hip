@@ -13,20 +13,29 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
   const int bk = kRowBytes / es;   // k values per K tile
   const int per16 = 16 / es;       // elements per 16 bytes
   if (a.bcols || a.ccols) return kUnsupported;
-  if (a.k % bk || a.k < bk) return kUnsupported;
-  // 128 x 128 when both extents allow, else the variant with one 64-wide side.
-  // With a K-contiguous B (op_b = N) n may be anything: the last tile column
-  // is masked.
+  if (a.k < bk) return kUnsupported;
+  // Extents need not be multiples of the tile: the last tile row / column and the last K tile are masked
+  // inside the kernel.  What must hold is that every run of elements that is contiguous in memory -- the
+  // rows of C and of a row-contiguous operand, K along a K-contiguous one -- is a whole number of 16-byte
+  // chunks, so that a chunk lies inside or outside the matrix.
   const bool any_n = a.op_b == GINN_HIP_OP_N;
-  int fm, fn;
-  if (a.m % 128 == 0 && a.n % 128 == 0) fm = 2, fn = 2;
-  else if (a.m % 128 == 0 && a.n % 64 == 0) fm = 2, fn = 1;
-  else if (a.m % 64 == 0 && a.n % 128 == 0) fm = 1, fn = 2;
-  // (A last tile column that is less than half full: 128 x 64 tiles for a narrow output, for which the
-  // wasted half tile counts; a wide one keeps 128 x 128 -- 4096 x 4000 x 4096 fp16: 194-221 us on 128 x 64.)
-  else if (any_n && a.m % 128 == 0) fm = 2, fn = (a.n <= 64 || ((a.n - 1) % 128 < 64 && a.n < 512)) ? 1 : 2;
-  else if (any_n && a.m % 64 == 0 && a.n > 64) fm = 1, fn = 2;
-  else return kUnsupported;
+  if (a.m % per16) return kUnsupported;
+  if (!any_n && a.n % per16) return kUnsupported;
+  if ((a.op_a == GINN_HIP_OP_T || any_n) && a.k % per16) return kUnsupported;
+  // 128 x 128 when both extents allow, else the variant with one 64-wide side.  A last tile row / column
+  // that is less than half full: the 64-wide side for a narrow output, for which the wasted half tile
+  // counts; a wide one keeps 128 (4096 x 4000 x 4096 fp16: 194-221 us on 128 x 64).
+  auto wide = [](int extent) {
+    if (extent % 128 == 0) return 2;
+    if (extent % 64 == 0) return 1;
+    return (extent <= 64 || ((extent - 1) % 128 < 64 && extent < 512)) ? 1 : 2;
+  };
+  int fm = wide(a.m), fn = wide(a.n);
+  // (Both sides 64 wide only by the tile counts below.)
+  if (fm == 1 && fn == 1) {
+    if (a.n > 64) fn = 2;
+    else if (a.m > 64) fm = 2;
+  }
   if (a.lda % per16 || a.ldb % per16 || a.ldc % per16) return kUnsupported;
   auto aligned16 = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
   if (!aligned16(a.A) || !aligned16(a.B) || !aligned16(a.C)) return kUnsupported;
@@ -51,15 +60,15 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
       // and no partial tiles to fold in a second launch (which costs what
       // some 20 K tiles of such a workgroup cost: the fewer the tiles, the
       // shorter the K up to which that holds).
-      const long long tiles64 = (long long)(a.m / 64) * ((a.n + 63) / 64) * a.batch;
-      const int kt = a.k / bk;
+      const long long tiles64 = (long long)((a.m + 63) / 64) * ((a.n + 63) / 64) * a.batch;
+      const int kt = (a.k + bk - 1) / bk;
       const bool enough = tiles64 >= ctx->num_cus || (tiles64 * 4 >= 3 * ctx->num_cus && kt <= 64) ||
                           (tiles64 * 8 >= 3 * ctx->num_cus && kt <= 32);
-      if (a.m % 64 == 0 && (a.n % 64 == 0 || any_n) && enough && tiles64 <= 2 * ctx->num_cus)
+      if (enough && tiles64 <= 2 * ctx->num_cus)
         fm = 1, fn = 1, f32_tiny_tiles = true;
       else if (fm == 2 && fn == 2) fn = 1;
-      const long long tiles = (long long)(a.m / (64 * fm)) * ((a.n + 64 * fn - 1) / (64 * fn)) * a.batch;
-      const long long by_k = a.batch == 1 ? std::max(1, (a.k / bk) / 2) : 1;
+      const long long tiles = (long long)((a.m + 64 * fm - 1) / (64 * fm)) * ((a.n + 64 * fn - 1) / (64 * fn)) * a.batch;
+      const long long by_k = a.batch == 1 ? std::max(1, kt / 2) : 1;
       if (tiles * by_k * 4 < ctx->num_cus) return kUnsupported;
     }
   }
@@ -72,9 +81,9 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
   // With a K-contiguous B the last tile column may be partly filled; the
   // narrowest right-hand sides (n <= 8, 4096 x n x 4096) stay 5 % faster on
   // 128 x 64 tiles.
-  if (!f32 && a.m % 64 == 0 && (a.n % 64 == 0 || (any_n && a.n > 8))) {
-    const long long tiles_now = (long long)(a.m / (64 * fm)) * ((a.n + 64 * fn - 1) / (64 * fn)) * a.batch;
-    const long long tiles64 = (long long)(a.m / 64) * ((a.n + 63) / 64) * a.batch;
+  if (!f32 && (a.n % 64 == 0 || a.n > 8)) {
+    const long long tiles_now = (long long)((a.m + 64 * fm - 1) / (64 * fm)) * ((a.n + 64 * fn - 1) / (64 * fn)) * a.batch;
+    const long long tiles64 = (long long)((a.m + 63) / 64) * ((a.n + 63) / 64) * a.batch;
     // (Two 64 x 64 workgroups per CU over a very long K run level with one 128-wide one:
     // 2048 x 1024 x 8192 49-57 against 51-52 us; those keep the larger shape.)
     if (tiles_now * 2 <= ctx->num_cus && !(tiles64 > ctx->num_cus && a.k / bk > 64)) fm = 1, fn = 1;
@@ -96,7 +105,7 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
   p.bias = a.bias;
   p.pre = a.pre;
   p.act = a.act;
-  p.tiles_m = a.m / (64 * fm);
+  p.tiles_m = (a.m + 64 * fm - 1) / (64 * fm);
   p.tiles_n = (a.n + 64 * fn - 1) / (64 * fn);
   p.partial = nullptr;
   const long long tiles = (long long)p.tiles_m * p.tiles_n;
@@ -104,7 +113,7 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
   if (p.group > p.tiles_m) p.group = p.tiles_m;
   const bool akc = a.op_a == GINN_HIP_OP_T;
   const bool bkc = a.op_b == GINN_HIP_OP_N;
-  const int kt_total = a.k / bk;
+  const int kt_total = (a.k + bk - 1) / bk;
 
   // Split K when the output has tiles for less than half of the CUs and K is
   // long: a split costs a second launch and moves its fp32 partial tiles

@@ -303,9 +303,11 @@ def test_seeded_random_shapes(dev, seed):
     from gpu_util import torch_dtype
     torch = dev.torch
     rng = random.Random(seed)
-    ms = [64, 128, 192, 256, 320, 384, 512, 640, 768, 1024, 1280, 1536, 2048, 2304, 3072, 4096, 100, 200, 1000, 33]
-    ns = ms + [1, 4, 8, 9, 16, 37, 40, 72, 130]
-    ks = [32, 64, 96, 128, 192, 256, 320, 512, 768, 1024, 1056, 1536, 2048, 2052, 3072, 4096, 100, 1000]
+    ms = [64, 128, 192, 256, 320, 384, 512, 640, 768, 1024, 1280, 1536, 2048, 2304, 3072, 4096, 100, 200, 1000, 33,
+          72, 136, 264, 520, 1032, 2056, 3080]
+    ns = ms + [1, 4, 8, 9, 16, 37, 40, 72, 130, 504]
+    ks = [32, 64, 96, 128, 192, 256, 320, 512, 768, 1024, 1056, 1536, 2048, 2052, 3072, 4096, 100, 1000,
+          72, 264, 328, 520, 4104]
     worst = {}
     for it in range(250):
         dt = rng.choice([capi.F32, capi.F16, capi.BF16])
@@ -411,3 +413,71 @@ def test_products_on_copies_keep_within_the_budget_for_temporaries(dev, dt, budg
     assert (took == 0) if budget is not None else (took >= 3), took
     err = float((C.double().transpose(1, 2) - want).norm() / want.norm())
     assert err <= 2 * _bound(dt), err
+
+
+def _masked_case(dev, dt, op_a, op_b, m, n, k, beta, batch=1):
+    """One product whose operands and result sit in buffers with 8 NaN-filled rows of padding below every
+    column (leading dimensions stay multiples of 8): a tile edge that reads beyond an extent shows up as
+    NaN in the result, and one that stores beyond it as a changed padding row."""
+    from gpu_util import round_to
+    rng = np.random.default_rng(m + 3 * n + 7 * k + op_a + 2 * op_b)
+    a_shape = (k, m) if op_a else (m, k)
+    b_shape = (n, k) if op_b else (k, n)
+    pad = 8
+    hs, bufs = [], []
+    for shape, scale in ((a_shape, 1 / np.sqrt(k)), (b_shape, 1.0), ((m, n), 1.0)):
+        h = round_to(rng.standard_normal(shape + (batch,)) * scale, dt)
+        hs.append(h)
+        bufs.append(dev.put(h.reshape(shape[0], -1, order="F"), dt, pad_rows=pad))
+    (A, B, C), ((ba, pa, lda), (bb, pb, ldb), (bc, pc, ldc)) = hs, bufs
+    es = 4 if dt == capi.F32 else 2
+    if batch == 1:
+        dev.gemm(dt, op_a, op_b, m, n, k, pa, lda, pb, ldb, beta, pc, ldc)
+    else:
+        dev.lib.call("ginn_hip_gemm_strided_batched", dev.ctx, dt, op_a, op_b, m, n, k, ctypes.c_void_p(pa), lda,
+                     lda * a_shape[1], ctypes.c_void_p(pb), ldb, ldb * b_shape[1], beta, ctypes.c_void_p(pc), ldc,
+                     ldc * n, batch)
+    dev.sync()
+    whole = bc.to(dev.torch.float32).cpu().numpy().reshape(batch * n, ldc)
+    assert np.isnan(whole[:, m:]).all(), "rows below the result were written"
+    got = whole[:, :m].reshape(batch, n, m).transpose(2, 1, 0)
+    assert not np.isnan(got).any(), "padding of an operand (or K beyond its end) reached the result"
+    for z in range(batch):
+        a64, b64 = A[..., z].astype(np.float64), B[..., z].astype(np.float64)
+        want = (a64.T if op_a else a64) @ (b64.T if op_b else b64) + beta * C[..., z].astype(np.float64)
+        err = np.linalg.norm(got[..., z] - want) / np.linalg.norm(want)
+        assert err <= 2 * _bound(dt), (z, err)
+    del es
+
+
+@pytest.mark.parametrize("dt", [capi.F16, capi.BF16, capi.F32])
+@pytest.mark.parametrize("op_a,op_b", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(136, 200, 72), (264, 72, 136), (520, 328, 1000), (1000, 1000, 1000),
+                                   (72, 1032, 264), (1288, 520, 96), (200, 2056, 3000)])
+@pytest.mark.parametrize("beta", [0.0, 0.5])
+def test_masked_tile_edges_of_the_128_wide_kernels(dev, dt, op_a, op_b, m, n, k, beta):
+    """Extents that are multiples of 8 but not of the tiles, leading dimensions that allow 16-byte accesses:
+    the last tile row, tile column and K tile are masked inside the tuned kernels (clamped loads, zeros
+    beyond K, masked stores) in every layout, as cuBLAS takes any m, n, k (ginn/prod.h:46-62).  The last
+    shape runs with K split over workgroups."""
+    _masked_case(dev, dt, op_a, op_b, m, n, k, beta)
+
+
+@pytest.mark.parametrize("dt", [capi.F16, capi.BF16])
+@pytest.mark.parametrize("op_a,op_b", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(3080, 3208, 264), (3848, 3976, 328), (4000, 4000, 1000)])
+@pytest.mark.parametrize("beta", [0.0, 0.5])
+def test_masked_tile_edges_of_the_256_wide_kernel(dev, dt, op_a, op_b, m, n, k, beta):
+    """The same on the 256 x 256 kernel (at least 144 tiles), plain and accumulating epilogue; the shapes
+    of the reference's own benchmark are 4000^3, 1000^3 and 16000 x 4000 (examples/bench.cu.cpp:216-220)."""
+    _masked_case(dev, dt, op_a, op_b, m, n, k, beta)
+
+
+@pytest.mark.parametrize("dt", [capi.F16, capi.BF16])
+@pytest.mark.parametrize("op_a,op_b,m,n,k", [(0, 0, 504, 504, 64), (0, 1, 504, 64, 504), (1, 0, 64, 504, 504),
+                                             (0, 0, 64, 504, 504), (0, 1, 64, 504, 504), (1, 0, 504, 504, 64),
+                                             (0, 0, 200, 64, 136), (1, 1, 72, 1000, 64)])
+def test_masked_tile_edges_of_the_small_slice_kernel(dev, dt, op_a, op_b, m, n, k):
+    """Attention products with a sequence length that is no multiple of 64 (T = 504, head size 64, 96
+    slices): forward and both gradients of Q K^T and P V, each slice's last tiles masked."""
+    _masked_case(dev, dt, op_a, op_b, m, n, k, 0.0, batch=96 if max(m, n, k) <= 504 else 40)
