@@ -51,6 +51,7 @@ def parse_args():
                    help="gemm (headline) | sweep (all GEMM shapes of the build target) | "
                         "configs (MLP, autobatched LSTM, attention products, GPT layer: GPU time with the CPU "
                         "oracle beside) | mlp | lstm | attention | gpt | update (one of those alone, for profiling) | "
+                        "ragged (products whose extents are no multiples of the tiles) | "
                         "copy (a plain copy kernel of known size, to calibrate the HBM counters)")
     p.add_argument("--dtype", default="f16", choices=list(DT))
     p.add_argument("--layout", default="NN", choices=["NN", "NT", "TN"])
@@ -319,20 +320,51 @@ def bench_attention(h, steps, warmup, cpu):
     return out
 
 
-def time_product(h, dtype, layout, m, n, k, steps, warmup):
+def time_product(h, dtype, layout, m, n, k, steps, warmup, batch=1):
     """Milliseconds per product (HIP events on the context's stream around back-to-back launches issued from
     native code, so that launches of a few microseconds are not bound by the interpreter); goes through
-    ginn_hip_gemm_strided_batched with one slice, which selects kernels exactly as ginn_hip_gemm does."""
-    A, B, C, lda, ldb = h.operands(dtype, layout, m, n, k)
+    ginn_hip_gemm_strided_batched, which with one slice selects kernels exactly as ginn_hip_gemm does."""
+    t = h.torch
+    g = t.Generator(device="cuda").manual_seed(0)
+    lda, a_cols = (k, m) if layout[0] == "T" else (m, k)
+    ldb, b_cols = (n, k) if layout[1] == "T" else (k, n)
+    A = (t.randn(batch, a_cols, lda, generator=g, device="cuda") / k ** 0.5).to(h.tdtype(dtype))
+    B = (t.randn(batch, b_cols, ldb, generator=g, device="cuda") / k ** 0.5).to(h.tdtype(dtype))
+    C = t.zeros(batch, n, m, device="cuda", dtype=h.tdtype(dtype))
+    t.cuda.synchronize()
     ex = _examples()
     ms = c_float(0)
     args = (h.ctx, DT[dtype], int(layout[0] == "T"), int(layout[1] == "T"), m, n, k, c_void_p(A.data_ptr()), lda,
-            ctypes.c_longlong(0), c_void_p(B.data_ptr()), ldb, ctypes.c_longlong(0), c_float(0.0),
-            c_void_p(C.data_ptr()), m, ctypes.c_longlong(0), 1)
+            ctypes.c_longlong(lda * a_cols), c_void_p(B.data_ptr()), ldb, ctypes.c_longlong(ldb * b_cols), c_float(0.0),
+            c_void_p(C.data_ptr()), m, ctypes.c_longlong(m * n), batch)
     for _ in range(2):  # the second measurement counts: the first meets clocks that are still moving
         if ex.scenario_time_batched_gemm(*args, warmup, steps, byref(ms)) != 0:
             raise SystemExit(f"scenario_time_batched_gemm: {ex.scenario_last_error().decode()}")
     return ms.value
+
+
+def bench_ragged(h, steps, warmup):
+    """Products whose extents are no multiples of the kernels' tiles: the shapes of the reference's own
+    benchmark (4000^3, 1000^3, 16000 x 16000 x 4000: examples/bench.cu.cpp:216-220), a vocabulary of 50 264
+    rows beside one of 50 304, and the attention products of a sequence length of 504 beside 512."""
+    cases = [("f16", "NN", 4000, 4000, 4000, 1), ("f16", "NT", 4000, 4000, 4000, 1), ("f16", "TN", 4000, 4000, 4000, 1),
+             ("f16", "NN", 4096, 4096, 4096, 1), ("f16", "NN", 2000, 2000, 2000, 1), ("f16", "NN", 1000, 1000, 1000, 1),
+             ("f16", "NN", 16000, 16000, 4000, 1), ("f32", "NN", 4000, 4000, 4000, 1), ("f32", "NN", 1000, 1000, 1000, 1),
+             ("bf16", "NN", 50264, 4096, 768, 1), ("bf16", "NN", 50304, 4096, 768, 1),
+             ("bf16", "NT", 50264, 768, 4096, 1), ("bf16", "NT", 50304, 768, 4096, 1),
+             ("bf16", "NN", 504, 504, 64, 96), ("bf16", "NN", 512, 512, 64, 96),
+             ("bf16", "NN", 64, 504, 504, 96), ("bf16", "NN", 64, 512, 512, 96),
+             ("bf16", "NT", 504, 64, 504, 96), ("bf16", "TN", 64, 504, 504, 96)]
+    time_product(h, "f16", "NN", 8192, 8192, 8192, 100, 100)  # untimed: lets the clocks settle
+    out = []
+    for dt, lay, m, n, k, batch in cases:
+        fl = 2.0 * m * n * k * batch
+        ms = time_product(h, dt, lay, m, n, k, max(5, min(steps, int(4e12 / fl) + 5)), warmup, batch)
+        by = ESIZE[dt] * (m * k + k * n + m * n) * batch
+        out.append({"config": f"{dt} {lay} {m}x{n}x{k}" + (f" x {batch} slices" if batch > 1 else ""),
+                    "us": round(ms * 1e3, 2), "tflops": round(fl / ms / 1e9, 1),
+                    "frac_mfma": round(fl / ms / 1e9 / PEAK_TFLOPS[dt], 4), "gbs": round(by / ms / 1e6, 1)})
+    return out
 
 
 def bench_update(h, steps, warmup, cpu):
@@ -549,6 +581,11 @@ def main():
         h.lib.call("ginn_hip_sync", h.ctx)
         print(json.dumps({"workload": "copy", "bytes_read_per_launch": a.size * a.size * ESIZE[a.dtype],
                           "bytes_written_per_launch": a.size * a.size * ESIZE[a.dtype]}))
+        return
+
+    if a.workload == "ragged":
+        for r in bench_ragged(h, max(1, a.steps), a.warmup):
+            print(json.dumps(r), flush=True)
         return
 
     if a.workload in ("configs", "mlp", "lstm", "attention", "gpt", "update"):

@@ -386,6 +386,12 @@ int ginn_hip_affine_bwd_pre(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
     bias_act = GINN_HIP_ACT_IDENTITY;
   }
 
+  // The kernel reads what the derivative is written in: the pre-activation (GELU, GELU2, LOG) or the
+  // output (the others), not both.
+  if (bias_act != GINN_HIP_ACT_IDENTITY) {
+    if (act_backward_requires_input(bias_act)) Y = nullptr;
+    else pre = nullptr;
+  }
   std::lock_guard<std::mutex> lock(ctx->mutex);
   const bool vec = vec8_ok({bias_src, Y, pre, dpre}, {static_cast<size_t>(m)});
   const rowred::Plan plan = rowred::plan(m, n, ctx->num_cus, ctx->workspace_bytes, 1, vec ? 8 : 1);

@@ -10,11 +10,25 @@
 namespace ginn {
 
 namespace internal {
+// The device type under which values of Scalar are MOVED, bit for bit: Int (indices, conditions) travels
+// as 4-byte words through the copies of the 4-byte floating type.  The layout nodes below are
+// instantiated and tested on Int in the reference (test/nodes.cu.cpp:66-306); their backward passes are
+// floating-point only.
+template <typename Scalar>
+inline ginn_hip_dtype move_dtype_of() {
+  if constexpr (is_floating_point_v<Scalar>) {
+    return dtype_of<Scalar>();
+  } else {
+    static_assert(sizeof(Scalar) == 4, "only 4-byte integers are moved as words");
+    return GINN_HIP_F32;
+  }
+}
 template <typename Scalar>
 void copy_2d(Tensor<Scalar>& dst, Size dst_off, Size ldd, const Tensor<Scalar>& src, Size src_off, Size lds,
              Size rows, Size cols, bool accumulate) {
   require_gpu(dst.dev(), "copy_2d");
-  GINN_HIP_CALL(ginn_hip_copy_2d(ctx_of(dst), dtype_of<Scalar>(), static_cast<int>(rows), static_cast<int>(cols),
+  GINN_ASSERT(!accumulate || is_floating_point_v<Scalar>, "only floating-point tensors are added to");
+  GINN_HIP_CALL(ginn_hip_copy_2d(ctx_of(dst), move_dtype_of<Scalar>(), static_cast<int>(rows), static_cast<int>(cols),
                                  src.data() + src_off, static_cast<int>(lds), dst.data() + dst_off,
                                  static_cast<int>(ldd), accumulate ? 1 : 0));
 }
@@ -22,7 +36,7 @@ void copy_2d(Tensor<Scalar>& dst, Size dst_off, Size ldd, const Tensor<Scalar>& 
 template <typename Scalar>
 LaunchDesc copy_desc(Scalar* dst, const Scalar* src, Size n, bool accumulate) {
   LaunchDesc d;
-  d.dtype = dtype_of<Scalar>();
+  d.dtype = move_dtype_of<Scalar>();  // (integer nodes describe nothing: they run their copies themselves)
   d.kind = GINN_HIP_MULTI_SUM;
   d.accumulate = accumulate;
   d.n = static_cast<size_t>(n);
@@ -92,7 +106,7 @@ class CatNode : public BaseDataNode<Scalar> {
   using BaseDataNode<Scalar>::grad;
   // Single-column inputs are contiguous pieces of the result.
   bool describe_forward(std::vector<LaunchDesc>& out) override {
-    if (value().dev()->kind() != GPU) return false;
+    if (value().dev()->kind() != GPU || !is_floating_point_v<Scalar>) return false;
     Size rows = 0;
     for (auto& in : ins_) {
       if (in->value().cols() != 1) return false;
@@ -107,7 +121,7 @@ class CatNode : public BaseDataNode<Scalar> {
     return true;
   }
   bool describe_backward(std::vector<LaunchDesc>& out) override {
-    if (value().dev()->kind() != GPU || value().cols() != 1) return false;
+    if (value().dev()->kind() != GPU || value().cols() != 1 || !is_floating_point_v<Scalar>) return false;
     Size at = 0;
     for (auto& in : ins_) {
       const Size r = in->value().rows();
@@ -166,7 +180,7 @@ class RowwiseCatNode : public BaseDataNode<Scalar>, public ColumnPartition {
   const std::vector<Size>& offsets() const override { return offsets_; }
   const std::vector<Size>& extents() const override { return extents_; }
   bool describe_forward(std::vector<LaunchDesc>& out) override {
-    if (value().dev()->kind() != GPU) return false;
+    if (value().dev()->kind() != GPU || !is_floating_point_v<Scalar>) return false;
     const Size rows = ins_[0]->value().rows();
     Size cols = 0;
     for (auto& in : ins_) {
@@ -187,7 +201,7 @@ class RowwiseCatNode : public BaseDataNode<Scalar>, public ColumnPartition {
     return true;
   }
   bool describe_backward(std::vector<LaunchDesc>& out) override {
-    if (value().dev()->kind() != GPU) return false;
+    if (value().dev()->kind() != GPU || !is_floating_point_v<Scalar>) return false;
     const Size rows = value().rows();
     Size at = 0;
     for (auto& in : ins_) {
@@ -363,7 +377,7 @@ class SliceNode : public BaseDataNode<Scalar> {
   // A window of whole columns, or inside a single column, is contiguous.
   bool contiguous(Size nr, Size nc) const { return nc == 1 || nr == in_->value().rows(); }
   bool describe_forward(std::vector<LaunchDesc>& out) override {
-    if (value().dev()->kind() != GPU || sizes_.size() > 2) return false;
+    if (value().dev()->kind() != GPU || sizes_.size() > 2 || !is_floating_point_v<Scalar>) return false;
     Size r0, c0, nr, nc;
     window(r0, c0, nr, nc);
     const Size rows = in_->value().rows();
@@ -375,7 +389,7 @@ class SliceNode : public BaseDataNode<Scalar> {
     return true;
   }
   bool describe_backward(std::vector<LaunchDesc>& out) override {
-    if (value().dev()->kind() != GPU || sizes_.size() > 2) return false;
+    if (value().dev()->kind() != GPU || sizes_.size() > 2 || !is_floating_point_v<Scalar>) return false;
     Size r0, c0, nr, nc;
     window(r0, c0, nr, nc);
     if (!contiguous(nr, nc)) return false;
@@ -428,6 +442,40 @@ class ReshapeNode : public BaseDataNode<Scalar> {
   std::string name() const override { return "Reshape"; }
 };
 GINN_MAKE_SCALAR_FORWARDING_FACTORY(Reshape);
+
+// The input under the shape that Tensor::reduce gives it for `rank` axes: trailing axes folded into the
+// last one kept, or axes of extent 1 appended (ginn/node/layout.h:529-561).  A view, like Reshape.
+template <typename Scalar>
+class RankViewNode : public BaseDataNode<Scalar> {
+  NodePtr<Scalar> in_;
+  Size rank_;
+
+  Shape view_shape() const { return Tensor<Scalar>::reduce(in_->shape(), rank_); }
+  void forward_() override { value().map(in_->value(), view_shape()); }
+
+ public:
+  using BaseDataNode<Scalar>::value;
+  GINN_GRAD_IS_VIEW_OF(in_)
+  bool has_grad() const override { return in_->has_grad(); }
+  void init_grad() override {
+    if (has_grad()) this->grad_storage().map(in_->grad_storage(), view_shape());
+  }
+  void reset_grad() override { init_grad(); }
+  bool describe_forward(std::vector<LaunchDesc>&) override {
+    forward_();
+    return true;
+  }
+  bool describe_backward(std::vector<LaunchDesc>&) override { return true; }
+  bool describe_reset_grad(std::vector<LaunchDesc>&) override {
+    init_grad();
+    return true;
+  }
+  RankViewNode(const NodePtr<Scalar>& x, Size rank) : BaseDataNode<Scalar>({x}), in_(x), rank_(rank) {
+    GINN_ASSERT(rank >= 1, "RankView: rank 0 is not handled (nor in ginn/node/layout.h:530)");
+  }
+  std::string name() const override { return "RankView"; }
+};
+GINN_MAKE_SCALAR_FORWARDING_FACTORY(RankView);
 
 // Identity view whose input can be rewired (ginn/node/layout.h:698-721); gives
 // Autobatch a consumer for nodes that otherwise end in non-rewirable users.
@@ -573,17 +621,19 @@ class ChipNode : public BaseDataNode<Scalar> {
     value().resize(s);
     Size inner, extent, outer;
     geometry(inner, extent, outer);
-    GINN_HIP_CALL(ginn_hip_copy_2d(internal::ctx_of(value()), dtype_of<Scalar>(), static_cast<int>(inner),
+    GINN_HIP_CALL(ginn_hip_copy_2d(internal::ctx_of(value()), internal::move_dtype_of<Scalar>(), static_cast<int>(inner),
                                    static_cast<int>(outer), in_->value().data() + offset_ * inner,
                                    static_cast<int>(inner * extent), value().data(), static_cast<int>(inner), 0));
   }
   void backward_() override {
     if (!in_->has_grad()) return;
-    Size inner, extent, outer;
-    geometry(inner, extent, outer);
-    GINN_HIP_CALL(ginn_hip_copy_2d(internal::ctx_of(grad()), dtype_of<Scalar>(), static_cast<int>(inner),
-                                   static_cast<int>(outer), grad().data(), static_cast<int>(inner),
-                                   in_->grad().data() + offset_ * inner, static_cast<int>(inner * extent), 1));
+    if constexpr (is_floating_point_v<Scalar>) {
+      Size inner, extent, outer;
+      geometry(inner, extent, outer);
+      GINN_HIP_CALL(ginn_hip_copy_2d(internal::ctx_of(grad()), dtype_of<Scalar>(), static_cast<int>(inner),
+                                     static_cast<int>(outer), grad().data(), static_cast<int>(inner),
+                                     in_->grad().data() + offset_ * inner, static_cast<int>(inner * extent), 1));
+    }
   }
 
  public:

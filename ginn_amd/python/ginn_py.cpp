@@ -256,6 +256,8 @@ void bind_float_nodes(py::module_& m) {
   m.def("AxisSum", [P](In x, const std::vector<Size>& axes) { return as_node(AxisSum(P(x), axes)); });
   m.def("Chip", [P](In x, Size offset, Size dim) { return as_node(Chip(P(x), offset, dim)); });
   m.def("Reshape", [P](In x, const Shape& s) { return as_node(Reshape(P(x), s)); });
+  m.def("RankView", [P](In x, Size rank) { return as_node(RankView(P(x), rank)); }, py::arg("in"), py::arg("rank"));
+  m.def("Slice", [P](In x, const Shape& offsets, const Shape& sizes) { return as_node(Slice(P(x), offsets, sizes)); });
   m.def("Permute", [P](In x, const Shape& s) { return as_node(Permute(P(x), s)); });
   m.def("Transpose", [P](In x, Size i, Size j) { return as_node(Transpose(P(x), i, j)); });
   m.def("RowBroadcast", [P](In x, Size rows) { return as_node(RowBroadcast(P(x), rows)); });

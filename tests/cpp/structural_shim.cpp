@@ -358,6 +358,98 @@ void arena_limits() {
   CHECK(reinterpret_cast<uintptr_t>(r.data()) % 256 == 0);
 }
 
+// The layout nodes on the HIP device with the known answers of test/nodes.cu.cpp:66-306 (Stack, Cat,
+// RowwiseCat / RowwiseUncat, Reshape, RankView, Slice, Chip), for the floating scalars and for Int, which
+// the reference instantiates them on as well.
+template <typename Scalar>
+Ptr<DataNode<Scalar>> on_gpu(const Ptr<DataNode<Real>>& x) {
+  auto y = x->template cast<Scalar>();
+  y->move_to(gpu());
+  y->set_has_grad(false);
+  return y;
+}
+
+template <typename Scalar, typename NodeT>
+void expect_values(int line, const Ptr<NodeT>& node, const Shape& shape, const std::vector<float>& want) {
+  Graph(node).forward();
+  if (node->shape() != shape) g_report += "line " + std::to_string(line) + ": unexpected shape\n";
+  const auto got = node->value().vector();
+  if (got.size() != want.size()) {
+    g_report += "line " + std::to_string(line) + ": unexpected size\n";
+    return;
+  }
+  for (size_t i = 0; i < got.size(); ++i)
+    if (static_cast<float>(got[i]) != want[i])
+      g_report += "line " + std::to_string(line) + ": element " + std::to_string(i) + " differs\n";
+}
+#define EXPECT_VALUES(node, shape, ...) expect_values<Scalar>(__LINE__, node, shape, std::vector<float> __VA_ARGS__)
+
+template <typename Scalar>
+void layout_goldens() {
+  using N = NodePtr<Scalar>;
+  {  // Stack of rank-1 (test/nodes.cu.cpp:69-88): result[x, i, j] = nodes[i][j][x], column-major storage
+    std::vector<N> v;
+    for (int b = 0; b < 6; ++b) v.push_back(on_gpu<Scalar>(Values<1>({1.f + 4 * b, 2.f + 4 * b, 3.f + 4 * b, 4.f + 4 * b})));
+    auto st = Stack<Scalar>({{v[0], v[1]}, {v[2], v[3]}, {v[4], v[5]}});
+    // element (x, i, j) at x + 4 (i + 3 j) holds nodes[i][j][x] = 1 + x + 4 (2 i + j)
+    std::vector<float> want(24);
+    for (int j = 0; j < 2; ++j)
+      for (int i = 0; i < 3; ++i)
+        for (int x = 0; x < 4; ++x) want[x + 4 * (i + 3 * j)] = 1.f + x + 4 * (2 * i + j);
+    expect_values<Scalar>(__LINE__, st, Shape{4, 3, 2}, want);
+    CHECK(want[4 * (1 + 3 * 0) + 0] == 9.f);   // the literal's entry [0][1][0]
+    CHECK(want[4 * (2 + 3 * 1) + 3] == 24.f);  // [3][2][1]
+  }
+  {  // Stack of rank-2 (:90-110)
+    std::vector<N> v;
+    for (int b = 0; b < 6; ++b)
+      v.push_back(on_gpu<Scalar>(Values<2>({{1.f + 4 * b, 2.f + 4 * b}, {3.f + 4 * b, 4.f + 4 * b}})));
+    auto st = Stack<Scalar>({{v[0], v[1]}, {v[2], v[3]}, {v[4], v[5]}});
+    std::vector<float> want(24);
+    for (int j = 0; j < 2; ++j)
+      for (int i = 0; i < 3; ++i)
+        for (int c = 0; c < 2; ++c)
+          for (int r = 0; r < 2; ++r) want[r + 2 * c + 4 * (i + 3 * j)] = 1.f + (2 * r + c) + 4 * (2 * i + j);
+    expect_values<Scalar>(__LINE__, st, Shape{2, 2, 3, 2}, want);
+  }
+  auto a12 = on_gpu<Scalar>(Values<2>({{1, 2}}));
+  auto b22 = on_gpu<Scalar>(Values<2>({{3, 4}, {5, 6}}));
+  auto c22 = on_gpu<Scalar>(Values<2>({{7, 8}, {9, 0}}));
+  // Cat (:126-148): rows on top of each other; column-major: 1 3 5 7 9 | 2 4 6 8 0
+  EXPECT_VALUES(Cat(N(a12), N(b22), N(c22)), (Shape{5, 2}), {1, 3, 5, 7, 9, 2, 4, 6, 8, 0});
+  {  // RowwiseCat (:151-199)
+    auto a = on_gpu<Scalar>(Values<2>({{1}, {2}}));
+    auto b = on_gpu<Scalar>(Values<2>({{3, 4}, {5, 6}}));
+    auto c = on_gpu<Scalar>(Values<2>({{7, 8, 9}, {0, 1, 2}}));
+    auto cat = RowwiseCat(N(a), N(b), N(c));
+    EXPECT_VALUES(cat, (Shape{2, 6}), {1, 2, 3, 5, 4, 6, 7, 0, 8, 1, 9, 2});
+    CHECK((cat->offsets() == std::vector<Size>{0, 1, 3}));
+    CHECK((cat->extents() == std::vector<Size>{1, 2, 3}));
+    EXPECT_VALUES(RowwiseUncat(N(cat), 0, cat), (Shape{2, 1}), {1, 2});
+    EXPECT_VALUES(RowwiseUncat(N(cat), 1, cat), (Shape{2, 2}), {3, 5, 4, 6});
+    EXPECT_VALUES(RowwiseUncat(N(cat), 2, cat), (Shape{2, 3}), {7, 0, 8, 1, 9, 2});
+  }
+  {  // Reshape (:202-223) and RankView (:226-251): the same storage under other shapes
+    auto W = on_gpu<Scalar>(Values<2>({{1, 2, 3, 4, 5, 6}}));
+    EXPECT_VALUES(Reshape(N(W), Shape{6, 1}), (Shape{6, 1}), {1, 2, 3, 4, 5, 6});
+    EXPECT_VALUES(Reshape(N(W), Shape{3, 2}), (Shape{3, 2}), {1, 2, 3, 4, 5, 6});
+    EXPECT_VALUES(Reshape(N(W), Shape{3, 1, 2}), (Shape{3, 1, 2}), {1, 2, 3, 4, 5, 6});
+    auto M = on_gpu<Scalar>(Values<2>({{1, 4}, {2, 5}, {3, 6}}));
+    EXPECT_VALUES(RankView(N(M), 1), (Shape{6}), {1, 2, 3, 4, 5, 6});
+    EXPECT_VALUES(RankView(N(M), 2), (Shape{3, 2}), {1, 2, 3, 4, 5, 6});
+    EXPECT_VALUES(RankView(N(M), 3), (Shape{3, 2, 1}), {1, 2, 3, 4, 5, 6});
+    CHECK_THROWS(RankView(N(M), 0));
+  }
+  {  // Slice (:254-286) and Chip (:288-306)
+    auto x = on_gpu<Scalar>(Values<2>({{1, 2}, {3, 4}, {5, 6}, {7, 8}}));
+    EXPECT_VALUES(Slice(N(x), Shape{1, 0}, Shape{3, 2}), (Shape{3, 2}), {3, 5, 7, 4, 6, 8});
+    EXPECT_VALUES(Slice(N(x), Shape{0, 1}, Shape{4, 1}), (Shape{4, 1}), {2, 4, 6, 8});
+    EXPECT_VALUES(Slice(N(x), Shape{2, 0}, Shape{2, 1}), (Shape{2, 1}), {5, 7});
+    EXPECT_VALUES(Chip(N(x), 2, 0), (Shape{2}), {5, 6});
+    EXPECT_VALUES(Chip(N(x), 1, 1), (Shape{4}), {2, 4, 6, 8});
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -392,6 +484,11 @@ const char* shim_structural(const char* which) {
       arena_nodes<Real>();
       arena_nodes<Half>();
       arena_nodes<BFloat16>();
+    } else if (w == "layout_goldens") {
+      layout_goldens<Real>();
+      layout_goldens<Half>();
+      layout_goldens<BFloat16>();
+      layout_goldens<Int>();
     } else if (w == "arena_limits") {
       arena_limits();
     } else {

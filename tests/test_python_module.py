@@ -237,6 +237,12 @@ def test_reference_python_cases(ginn, scalar_name):
     lt = W < (W * 0 + 3.5)
     ginn.Graph(lt).forward()
     assert lt.value.list() == [True, False, True, False, True, False]
+    # test_rank_view of ginn-py/test/test_nodes.py:183-201 and its neighbours Reshape / Slice
+    M = ginn.Values(dev, [[1, 4], [2, 5], [3, 6]]).cast(scalar)
+    check(ginn.RankView(M, 1), ginn.Values(dev, [1, 2, 3, 4, 5, 6]).cast(scalar), aeps)
+    check(ginn.RankView(M, 2), M, aeps)
+    check(ginn.RankView(M, 3), ginn.Values(dev, [[[1], [4]], [[2], [5]], [[3], [6]]]).cast(scalar), aeps)
+    check(ginn.Slice(M, [1, 0], [2, 2]), ginn.Values(dev, [[2, 5], [3, 6]]).cast(scalar), aeps)
 
 
 @pytest.mark.gpu

@@ -20,6 +20,7 @@ CASES = [
     (capi.F32, [(4096, 1, 4096), (512, 64, 784)]),       # vector skinny kernel; generic kernel with split-K
     (capi.F16, [(4096, 4, 8192), (2048, 1, 4096)]),      # 16-bit skinny kernel
     (capi.BF16, [(768, 768, 4096), (256, 128, 2048)]),   # 128 x 128 family with split-K
+    (capi.F16, [(1000, 1000, 1000), (200, 136, 72)]),    # masked tile edges (no copies, no cuts)
 ]
 
 
