@@ -425,6 +425,7 @@ int launch_gemm_ksplit(ginn_hip_ctx* ctx, const GemmArgs& args);
 
 // Bandwidth-oriented kernel for narrow right-hand sides (n <= 64).
 int launch_gemm_skinny(ginn_hip_ctx* ctx, const GemmArgs& args);
+int launch_gemm_strip(ginn_hip_ctx* ctx, const GemmArgs& args);
 int launch_gemm_skinny_mfma(ginn_hip_ctx* ctx, const GemmArgs& args);
 // 16-bit, 128 x 128 x 64 tiles with optional split-K: aligned shapes whose
 // 256 x 256 tiling would leave most CUs idle; kUnsupported otherwise.

@@ -272,7 +272,8 @@ int launch_gemm(ginn_hip_ctx* ctx, const GemmArgs& a) {
   // the vector-ALU kernel and has the arithmetic for free (fp16 4096 x n x 4096: 7.9-8.5 us for n = 1 .. 8
   // against 8.5-15.2 us); the vector-ALU kernel keeps fp32 (whose matrix pipe is 16 x slower) and the 16-bit
   // shapes the matrix-core kernel does not take (unaligned operands, odd extents).
-  int rc = kUnsupported;
+  int rc = launch_gemm_strip(ctx, a);
+  if (rc != kUnsupported) return rc;
   if (a.dtype != GINN_HIP_F32 && a.batch == 1 && a.n <= 8) rc = launch_gemm_mid(ctx, a);
   if (rc != kUnsupported) return rc;
   rc = launch_gemm_ksplit(ctx, a);

@@ -80,6 +80,8 @@ def test_reference_affine_goldens(dev, golden, dt):
                                    (384, 128, 2048, 0), (3072, 4096, 256, 0), (1024, 1, 384, 0),
                                    (2048, 8, 640, 64), (256, 64, 128, 0), (64, 256, 256, 64), (512, 40, 192, 0),
                                    (1024, 512, 256, 64),
+                                   # tall A, at most 16 columns, long K: one launch of 16-row strips, fused epilogue
+                                   (2048, 5, 1024, 1040), (4104, 16, 1040, 0),
                                    # odd leading dimensions, large: the products run on padded copies
                                    (1001, 1003, 1005, 0), (1501, 1503, 1505, 515)])
 def test_affine_forward(dev, dt, act, shape):

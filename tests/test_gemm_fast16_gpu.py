@@ -481,3 +481,17 @@ def test_masked_tile_edges_of_the_small_slice_kernel(dev, dt, op_a, op_b, m, n, 
     """Attention products with a sequence length that is no multiple of 64 (T = 504, head size 64, 96
     slices): forward and both gradients of Q K^T and P V, each slice's last tiles masked."""
     _masked_case(dev, dt, op_a, op_b, m, n, k, 0.0, batch=96 if max(m, n, k) <= 504 else 40)
+
+
+@pytest.mark.parametrize("dt", [capi.F16, capi.BF16, capi.F32])
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 8, 9, 16])
+@pytest.mark.parametrize("m,k", [(2048, 1024), (4096, 4096), (2056, 1040), (4104, 2064), (2048, 8208), (4096, 1040),
+                                 (4104, 1056)])
+@pytest.mark.parametrize("beta", [0.0, 0.5])
+def test_narrow_right_hand_sides_in_one_launch(dev, dt, n, m, k, beta):
+    """NN products with at most 16 columns over a tall A of up to 24 MiB (fp32: 8 .. 16 columns, up to 32 MiB)
+    run as one launch of 16-row strips over all of K (gemm_strip.hip; the degenerate end of
+    ginn/prod.h:32-66), larger ones on the kernels that split K over workgroups: every width of the B
+    loads (n <= 4, 8, 16), a last strip that is partly filled, K ranges that split unevenly over the four
+    waves and buffers that are partly used, plain and accumulating epilogue, NaN padding around every operand."""
+    _masked_case(dev, dt, 0, 0, m, n, k, beta)
