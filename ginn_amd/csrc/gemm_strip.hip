@@ -22,7 +22,10 @@
 //
 // What it reaches (fp16 4096 x 1 x 4096, kernel alone): 5.9 us with the loads of A only, 6.3 with the
 // epilogue, 7.6 with the loads of B (one more load instruction in five), 8.5 us with operand reads and
-// MFMAs -- level with the two launches of the split kernels at that size, ahead below it.
+// MFMAs -- level with the two launches of the split kernels at that size, ahead below it.  The loads alone are
+// bound by what a CU's first-level cache takes in: it fetches whole 128-byte lines of which the strip uses a
+// quarter, 512 KiB per CU for this A, the same as with full lines on a quarter of the CUs.  (A vector-ALU form
+// for n <= 4 with B in LDS as fp32 was measured too: 13.6 us, unpacking and multiplying 16-bit rows one by one.)
 #include <type_traits>
 
 #include "common.h"
@@ -371,3 +374,4 @@ int launch_gemm_strip(ginn_hip_ctx* ctx, const GemmArgs& a) {
 }
 
 }  // namespace ginn_hip
+
