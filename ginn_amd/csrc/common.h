@@ -423,6 +423,12 @@ int launch_gemm_fast16(ginn_hip_ctx* ctx, const GemmArgs& args);
 // the 16 waves of a workgroup, one launch; kUnsupported otherwise.
 int launch_gemm_ksplit(ginn_hip_ctx* ctx, const GemmArgs& args);
 
+// Element-wise arithmetic on 32-bit integer tensors (GINN_HIP_I32), exact: dst (+)= op(a, b, c).
+// kIntAdd: a + b (b may be NULL); kIntScaleShift: ia * a + ib; kIntMulAdd: a (*) (b + ia) + c with b and c
+// indexed per row (i % rows) when rows != 0.
+enum IntOp { kIntAdd = 0, kIntSub, kIntMul, kIntMax, kIntScaleShift, kIntMulAdd };
+int launch_int_arith(ginn_hip_ctx* ctx, int op, size_t n, size_t rows, const void* a, const void* b, const void* c,
+                     int ia, int ib, void* dst, int accumulate);
 // Bandwidth-oriented kernel for narrow right-hand sides (n <= 64).
 int launch_gemm_skinny(ginn_hip_ctx* ctx, const GemmArgs& args);
 int launch_gemm_strip(ginn_hip_ctx* ctx, const GemmArgs& args);

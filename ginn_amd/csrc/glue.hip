@@ -397,6 +397,14 @@ int ginn_hip_add_n(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n, int count,
     GH_CHECK_ARG(host_srcs[k], "ginn_hip_add_n: source %d is NULL", k);
     srcs.p[k] = host_srcs[k];
   }
+  if (dtype == GINN_HIP_I32) {  // two sources per launch
+    for (int k = 0; k < count; k += 2) {
+      const int rc = launch_int_arith(ctx, kIntAdd, n, 0, host_srcs[k], k + 1 < count ? host_srcs[k + 1] : nullptr,
+                                      nullptr, 0, 0, dst, (accumulate || k > 0) ? 1 : 0);
+      if (rc != kOk) return rc;
+    }
+    return kOk;
+  }
   GH_HIP(hipSetDevice(ctx->device));
   bool vec = vec8_ok({dst}, {n});
   for (int k = 0; k < count; ++k) vec = vec && vec8_ok({host_srcs[k]}, {});
@@ -411,6 +419,7 @@ int ginn_hip_cwise_prod(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n, const
   GH_CHECK_ARG(ctx, "ginn_hip_cwise_prod: ctx is NULL");
   if (n == 0) return kOk;
   GH_CHECK_ARG(a && b && dst, "ginn_hip_cwise_prod: NULL pointer");
+  if (dtype == GINN_HIP_I32) return launch_int_arith(ctx, kIntMul, n, 0, a, b, nullptr, 0, 0, dst, accumulate);
   GH_HIP(hipSetDevice(ctx->device));
   const bool vec = vec8_ok({a, b, dst}, {n});
   const unsigned grid = grid_for(vec ? n / 8 : n, kBlock, ctx->num_cus);
@@ -425,6 +434,9 @@ int ginn_hip_scale_shift(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n, floa
   GH_CHECK_ARG(ctx, "ginn_hip_scale_shift: ctx is NULL");
   if (n == 0) return kOk;
   GH_CHECK_ARG(x && dst, "ginn_hip_scale_shift: NULL pointer");
+  if (dtype == GINN_HIP_I32)
+    return launch_int_arith(ctx, kIntScaleShift, n, 0, x, nullptr, nullptr, static_cast<int>(alpha),
+                            static_cast<int>(shift), dst, accumulate);
   GH_HIP(hipSetDevice(ctx->device));
   const bool vec = vec8_ok({x, dst}, {n});
   const unsigned grid = grid_for(vec ? n / 8 : n, kBlock, ctx->num_cus);

@@ -417,11 +417,17 @@ extern "C" {
 
 int ginn_hip_elementwise(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, ginn_hip_ew_op op, size_t n, const void* a,
                          const void* b, const void* c, void* dst, int accumulate) {
-  GH_ENTER("ginn_hip_elementwise", ctx);
+  GH_CHECK_ARG(ctx, "ginn_hip_elementwise: ctx is NULL");
+  GH_CHECK_ARG(dtype_valid(dtype) || dtype == GINN_HIP_I32, "ginn_hip_elementwise: unknown dtype %d", dtype);
   GH_CHECK_ARG(op >= GINN_HIP_EW_SUB && op <= GINN_HIP_EW_DIV_MUL, "ginn_hip_elementwise: unknown op %d", op);
   if (n == 0) return kOk;
   const bool three = op == GINN_HIP_EW_EQ_MUL || op == GINN_HIP_EW_DIV_MUL;
   GH_CHECK_ARG(a && b && dst && (!three || c), "ginn_hip_elementwise: NULL operand");
+  if (dtype == GINN_HIP_I32) {
+    GH_CHECK_ARG(!three, "ginn_hip_elementwise: operation %d has no integer form", op);
+    return launch_int_arith(ctx, op == GINN_HIP_EW_SUB ? kIntSub : kIntMax, n, 0, a, b, nullptr, 0, 0, dst,
+                            accumulate);
+  }
   GH_HIP(hipSetDevice(ctx->device));
   const bool vec = vec8_ok({a, b, c, dst}, {n});
   const unsigned grid = grid_for(vec ? n / 8 : n, kBlock, ctx->num_cus);

@@ -644,6 +644,9 @@ int ginn_hip_cwise_prod_add_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int row
   GH_CHECK_ARG(rows >= 0 && cols >= 0, "ginn_hip_cwise_prod_add_fwd: negative dimension");
   if (rows == 0 || cols == 0) return kOk;
   GH_CHECK_ARG(a && b && c && y, "ginn_hip_cwise_prod_add_fwd: NULL pointer");
+  if (dtype == GINN_HIP_I32)
+    return launch_int_arith(ctx, kIntMulAdd, static_cast<size_t>(rows) * cols, broadcast ? static_cast<size_t>(rows) : 0,
+                            a, b, c, static_cast<int>(multiplier_bias), 0, y, 0);
   GH_HIP(hipSetDevice(ctx->device));
   const size_t n = static_cast<size_t>(rows) * cols;
   const bool vec = vec8_ok({a, b, c, y}, {static_cast<size_t>(rows)});

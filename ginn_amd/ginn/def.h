@@ -127,6 +127,15 @@ inline ginn_hip_dtype dtype_of() {
   return GINN_HIP_BF16;
 }
 
+// The same for the nodes that exist on Int as well (ginn/node/common.h: Add, Subtract, the scalar forms,
+// CwiseProd, CwiseProdAdd, CwiseMax): their forward passes take GINN_HIP_I32, exact integer arithmetic;
+// Int nodes carry no gradient.
+template <typename Scalar>
+inline ginn_hip_dtype arith_dtype_of() {
+  if constexpr (std::is_same_v<Scalar, Int>) return GINN_HIP_I32;
+  else return dtype_of<Scalar>();
+}
+
 namespace literals {
 inline Real operator"" _r(long double x) { return static_cast<Real>(x); }
 inline Real operator"" _r(unsigned long long x) { return static_cast<Real>(x); }

@@ -24,7 +24,7 @@ void add_tensors(Tensor<Scalar>& dst, const std::vector<const Tensor<Scalar>*>& 
       GINN_ASSERT(srcs[i + k]->size() == dst.size(), "Add: operand sizes differ");
       p[k] = srcs[i + k]->data();
     }
-    GINN_HIP_CALL(ginn_hip_add_n(ctx_of(dst), dtype_of<Scalar>(), n, count, p, dst.data(),
+    GINN_HIP_CALL(ginn_hip_add_n(ctx_of(dst), arith_dtype_of<Scalar>(), n, count, p, dst.data(),
                                  (accumulate || i > 0) ? 1 : 0));
   }
 }
@@ -58,11 +58,11 @@ class AddNode : public BaseDataNode<Scalar> {
   BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; }
 
   bool describe_forward(std::vector<LaunchDesc>& out) override {
-    if (value().dev()->kind() != GPU) return false;
+    if (value().dev()->kind() != GPU || !is_floating_point_v<Scalar>) return false;
     value().resize(ins_[0]->value().shape());
     for (size_t i = 0; i < ins_.size(); i += 3) {
       LaunchDesc d;
-      d.dtype = dtype_of<Scalar>();
+      d.dtype = arith_dtype_of<Scalar>();
       d.kind = GINN_HIP_MULTI_SUM;
       d.accumulate = i > 0;
       d.n = static_cast<size_t>(value().size());
@@ -76,11 +76,11 @@ class AddNode : public BaseDataNode<Scalar> {
     return true;
   }
   bool describe_backward(std::vector<LaunchDesc>& out) override {
-    if (value().dev()->kind() != GPU) return false;
+    if (value().dev()->kind() != GPU || !is_floating_point_v<Scalar>) return false;
     for (auto& in : ins_) {
       if (!in->has_grad()) continue;
       LaunchDesc d;
-      d.dtype = dtype_of<Scalar>();
+      d.dtype = arith_dtype_of<Scalar>();
       d.kind = GINN_HIP_MULTI_SUM;
       d.accumulate = !in->take_lazy_zero();
       d.n = static_cast<size_t>(grad().size());
@@ -111,7 +111,7 @@ class CwiseProdNode : public BaseDataNode<Scalar> {
 
   void run(Tensor<Scalar>& dst, const Tensor<Scalar>& x, const Tensor<Scalar>& y, bool acc) {
     internal::require_gpu(dst.dev(), "CwiseProd");
-    GINN_HIP_CALL(ginn_hip_cwise_prod(internal::ctx_of(dst), dtype_of<Scalar>(), static_cast<size_t>(dst.size()),
+    GINN_HIP_CALL(ginn_hip_cwise_prod(internal::ctx_of(dst), arith_dtype_of<Scalar>(), static_cast<size_t>(dst.size()),
                                       x.data(), y.data(), dst.data(), acc ? 1 : 0));
   }
   void forward_() override {
@@ -136,7 +136,7 @@ class CwiseProdNode : public BaseDataNode<Scalar> {
   BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; }
   LaunchDesc prod_desc(Scalar* dst, const Scalar* x, const Scalar* y, bool accumulate) const {
     LaunchDesc d;
-    d.dtype = dtype_of<Scalar>();
+    d.dtype = arith_dtype_of<Scalar>();
     d.kind = GINN_HIP_MULTI_PROD;
     d.accumulate = accumulate;
     d.n = static_cast<size_t>(value().size());
@@ -146,14 +146,14 @@ class CwiseProdNode : public BaseDataNode<Scalar> {
     return d;
   }
   bool describe_forward(std::vector<LaunchDesc>& out) override {
-    if (value().dev()->kind() != GPU) return false;
+    if (value().dev()->kind() != GPU || !is_floating_point_v<Scalar>) return false;
     GINN_ASSERT(a_->value().size() == b_->value().size(), "CwiseProd: operand sizes differ");
     value().resize(a_->value().shape());
     out.push_back(prod_desc(value().data(), a_->value().data(), b_->value().data(), false));
     return true;
   }
   bool describe_backward(std::vector<LaunchDesc>& out) override {
-    if (value().dev()->kind() != GPU) return false;
+    if (value().dev()->kind() != GPU || !is_floating_point_v<Scalar>) return false;
     if (a_->has_grad()) {
       const bool fresh = a_->take_lazy_zero();
       out.push_back(prod_desc(a_->grad().data(), grad().data(), b_->value().data(), !fresh));
@@ -187,14 +187,14 @@ class ScaleShiftNode : public BaseDataNode<Scalar> {
   void forward_() override {
     internal::require_gpu(this->dev(), name_);
     value().resize(in_->value().shape());
-    GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(value()), dtype_of<Scalar>(),
+    GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(value()), arith_dtype_of<Scalar>(),
                                        static_cast<size_t>(value().size()), alpha_, shift_, in_->value().data(),
                                        value().data(), 0));
   }
   void backward_() override {
     if (!in_->has_grad()) return;
     const bool fresh = in_->take_lazy_zero();
-    GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(grad()), dtype_of<Scalar>(),
+    GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(grad()), arith_dtype_of<Scalar>(),
                                        static_cast<size_t>(grad().size()), alpha_, 0.f, grad().data(),
                                        in_->grad().data(), fresh ? 0 : 1));
   }
@@ -236,13 +236,13 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
       ln->pending_ = false;
       auto& x = ln->in_->value();
       GINN_HIP_CALL(ginn_hip_layernorm_affine_fwd(
-          internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()), static_cast<int>(x.cols()), x.data(),
+          internal::ctx_of(x), arith_dtype_of<Scalar>(), static_cast<int>(x.rows()), static_cast<int>(x.cols()), x.data(),
           ln->eps_, b_->value().data(), c_->value().data(), multiplier_bias_, ln->raw_value().data(), ln->std_.data(),
           value().data()));
       return;
     }
     auto& a = a_->value();
-    GINN_HIP_CALL(ginn_hip_cwise_prod_add_fwd(internal::ctx_of(a), dtype_of<Scalar>(), static_cast<int>(a.rows()),
+    GINN_HIP_CALL(ginn_hip_cwise_prod_add_fwd(internal::ctx_of(a), arith_dtype_of<Scalar>(), static_cast<int>(a.rows()),
                                               static_cast<int>(a.cols()), a.data(), b_->value().data(),
                                               c_->value().data(), multiplier_bias_, broadcast_ ? 1 : 0,
                                               value().data()));
@@ -259,7 +259,7 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
       auto& x = ln->in_;
       const bool x_fresh = x->has_grad() && x->take_lazy_zero();
       GINN_HIP_CALL(ginn_hip_layernorm_affine_bwd(
-          internal::ctx_of(a), dtype_of<Scalar>(), static_cast<int>(a.rows()), static_cast<int>(a.cols()),
+          internal::ctx_of(a), arith_dtype_of<Scalar>(), static_cast<int>(a.rows()), static_cast<int>(a.cols()),
           grad().data(), a.data(), ln->std_.data(), b_->value().data(), multiplier_bias_,
           x->has_grad() ? x->grad().data() : nullptr, x_fresh ? 0 : 1, b_->has_grad() ? b_->grad().data() : nullptr,
           c_->has_grad() ? c_->grad().data() : nullptr));
@@ -267,15 +267,19 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
       return;
     }
     GINN_HIP_CALL((fresh ? ginn_hip_cwise_prod_add_bwd_assign : ginn_hip_cwise_prod_add_bwd)(
-        internal::ctx_of(a), dtype_of<Scalar>(), static_cast<int>(a.rows()), static_cast<int>(a.cols()),
+        internal::ctx_of(a), arith_dtype_of<Scalar>(), static_cast<int>(a.rows()), static_cast<int>(a.cols()),
         grad().data(), a.data(), b_->value().data(), multiplier_bias_, broadcast_ ? 1 : 0,
         a_->has_grad() ? a_->grad().data() : nullptr, b_->has_grad() ? b_->grad().data() : nullptr,
         c_->has_grad() ? c_->grad().data() : nullptr));
   }
   // The LayerNorm this node follows directly, if any (not one that normalises in place).
   LayerNormNode<Scalar>* layer_norm() const {
-    auto* ln = dynamic_cast<LayerNormNode<Scalar>*>(a_.get());
-    return ln && ln->may_postpone() ? ln : nullptr;
+    if constexpr (is_floating_point_v<Scalar>) {
+      auto* ln = dynamic_cast<LayerNormNode<Scalar>*>(a_.get());
+      return ln && ln->may_postpone() ? ln : nullptr;
+    } else {
+      return nullptr;
+    }
   }
 
  public:
@@ -326,14 +330,14 @@ class SubtractNode : public BaseDataNode<Scalar> {
     internal::require_gpu(this->dev(), "Subtract");
     GINN_ASSERT(left_->value().size() == right_->value().size(), "Subtract: operand sizes differ");
     value().resize(left_->value().shape());
-    GINN_HIP_CALL(ginn_hip_elementwise(internal::ctx_of(value()), dtype_of<Scalar>(), GINN_HIP_EW_SUB,
+    GINN_HIP_CALL(ginn_hip_elementwise(internal::ctx_of(value()), arith_dtype_of<Scalar>(), GINN_HIP_EW_SUB,
                                        static_cast<size_t>(value().size()), left_->value().data(),
                                        right_->value().data(), nullptr, value().data(), 0));
   }
   void backward_() override {
     if (left_->has_grad()) internal::add_tensors(left_->grad(), {&grad()}, true);
     if (right_->has_grad())
-      GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(grad()), dtype_of<Scalar>(),
+      GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(grad()), arith_dtype_of<Scalar>(),
                                          static_cast<size_t>(grad().size()), -1.f, 0.f, grad().data(),
                                          right_->grad().data(), 1));
   }
@@ -358,7 +362,7 @@ class CwiseMaxNode : public BaseDataNode<Scalar> {
     value() = ins_[0]->value();
     for (size_t i = 1; i < ins_.size(); ++i) {
       GINN_ASSERT(ins_[i]->value().size() == value().size(), "CwiseMax: operand sizes differ");
-      GINN_HIP_CALL(ginn_hip_elementwise(internal::ctx_of(value()), dtype_of<Scalar>(), GINN_HIP_EW_MAX,
+      GINN_HIP_CALL(ginn_hip_elementwise(internal::ctx_of(value()), arith_dtype_of<Scalar>(), GINN_HIP_EW_MAX,
                                          static_cast<size_t>(value().size()), value().data(),
                                          ins_[i]->value().data(), nullptr, value().data(), 0));
     }
@@ -366,7 +370,7 @@ class CwiseMaxNode : public BaseDataNode<Scalar> {
   void backward_() override {
     for (auto& in : ins_)
       if (in->has_grad())
-        GINN_HIP_CALL(ginn_hip_elementwise(internal::ctx_of(grad()), dtype_of<Scalar>(), GINN_HIP_EW_EQ_MUL,
+        GINN_HIP_CALL(ginn_hip_elementwise(internal::ctx_of(grad()), arith_dtype_of<Scalar>(), GINN_HIP_EW_EQ_MUL,
                                            static_cast<size_t>(grad().size()), grad().data(), in->value().data(),
                                            value().data(), in->grad().data(), 1));
   }

@@ -211,6 +211,38 @@ void bind_node_types(py::module_& m) {
   }
 }
 
+// The nodes that exist for Int as well as for the floating scalars (ginn-py/node/common-py.cu.cpp:34-70,
+// ginn-py/node/layout-py.cu.cpp): arithmetic, layout, comparison.
+template <typename S>
+void bind_shared_nodes(py::module_& m) {
+  using N = Node<S>;
+  using In = const SP<N>&;
+  auto P = [](In x) { return NodePtr<S>(x); };
+  m.def("Add", [](const std::vector<SP<N>>& ins) { return as_node(Add(ptrs<S>(ins))); });
+  m.def("Add", [P](In a, In b) { return as_node(Add(P(a), P(b))); });
+  m.def("Subtract", [P](In a, In b) { return as_node(Subtract(P(a), P(b))); });
+  m.def("CwiseProd", [P](In a, In b) { return as_node(CwiseProd(P(a), P(b))); });
+  m.def("CwiseMax", [](const std::vector<SP<N>>& ins) { return as_node(CwiseMax(ptrs<S>(ins))); });
+  m.def("CwiseProdAdd",
+        [P](In a, In b, In c, double bias) { return as_node(CwiseProdAdd(P(a), P(b), P(c), S(static_cast<float>(bias)))); },
+        py::arg("a"), py::arg("b"), py::arg("c"), py::arg("multiplier_bias") = 0.);
+  m.def("AddScalar", [P](In x, double s) { return as_node(AddScalar(P(x), s)); });
+  m.def("SubtractScalar", [P](double s, In x) { return as_node(SubtractScalar(s, P(x))); });
+  m.def("ProdScalar", [P](In x, double s) { return as_node(ProdScalar(P(x), s)); });
+  m.def("Chip", [P](In x, Size offset, Size dim) { return as_node(Chip(P(x), offset, dim)); });
+  m.def("Reshape", [P](In x, const Shape& s) { return as_node(Reshape(P(x), s)); });
+  m.def("RankView", [P](In x, Size rank) { return as_node(RankView(P(x), rank)); }, py::arg("in"), py::arg("rank"));
+  m.def("Slice", [P](In x, const Shape& offsets, const Shape& sizes) { return as_node(Slice(P(x), offsets, sizes)); });
+  m.def("Cat", [](const std::vector<SP<N>>& ins) { return as_node(Cat(ptrs<S>(ins))); });
+  m.def("RowwiseCat", [](const std::vector<SP<N>>& ins) { return as_node(RowwiseCat(ptrs<S>(ins))); });
+  m.def("Stack", [](const std::vector<std::vector<SP<N>>>& grid) {
+    std::vector<std::vector<NodePtr<S>>> g;
+    for (auto& row : grid) g.push_back(ptrs<S>(row));
+    return as_node(Stack<S>(g));
+  });
+  m.def("LessThan", [P](In a, In b) { return SP<Node<bool>>(LessThan(P(a), P(b)).as_shared_ptr()); });
+}
+
 // Everything that computes, for one floating scalar type: overloads of the
 // same Python name are told apart by the node type of their arguments.
 template <typename S>
@@ -226,17 +258,7 @@ void bind_float_nodes(py::module_& m) {
           return as_node(make_ptr<AffineNode<S>>(nonlin_by_name<S>(nonlin), ptrs<S>(ins)));
         },
         py::arg("ins"), py::arg("nonlin") = "identity");
-  m.def("Add", [](const std::vector<SP<N>>& ins) { return as_node(Add(ptrs<S>(ins))); });
-  m.def("Add", [P](In a, In b) { return as_node(Add(P(a), P(b))); });
-  m.def("Subtract", [P](In a, In b) { return as_node(Subtract(P(a), P(b))); });
-  m.def("CwiseProd", [P](In a, In b) { return as_node(CwiseProd(P(a), P(b))); });
-  m.def("CwiseMax", [](const std::vector<SP<N>>& ins) { return as_node(CwiseMax(ptrs<S>(ins))); });
-  m.def("CwiseProdAdd",
-        [P](In a, In b, In c, double bias) { return as_node(CwiseProdAdd(P(a), P(b), P(c), S(static_cast<float>(bias)))); },
-        py::arg("a"), py::arg("b"), py::arg("c"), py::arg("multiplier_bias") = 0.);
-  m.def("AddScalar", [P](In x, double s) { return as_node(AddScalar(P(x), s)); });
-  m.def("SubtractScalar", [P](double s, In x) { return as_node(SubtractScalar(s, P(x))); });
-  m.def("ProdScalar", [P](In x, double s) { return as_node(ProdScalar(P(x), s)); });
+  bind_shared_nodes<S>(m);
   m.def("Dropout", [P](In x, double p) { return as_node(Dropout(P(x), static_cast<Real>(p))); });
 #define GINN_PY_UNARY(F) m.def(#F, [P](In x) { return as_node(F(P(x))); })
   GINN_PY_UNARY(Identity);
@@ -254,24 +276,12 @@ void bind_float_nodes(py::module_& m) {
   GINN_PY_UNARY(LayerNorm);
 #undef GINN_PY_UNARY
   m.def("AxisSum", [P](In x, const std::vector<Size>& axes) { return as_node(AxisSum(P(x), axes)); });
-  m.def("Chip", [P](In x, Size offset, Size dim) { return as_node(Chip(P(x), offset, dim)); });
-  m.def("Reshape", [P](In x, const Shape& s) { return as_node(Reshape(P(x), s)); });
-  m.def("RankView", [P](In x, Size rank) { return as_node(RankView(P(x), rank)); }, py::arg("in"), py::arg("rank"));
-  m.def("Slice", [P](In x, const Shape& offsets, const Shape& sizes) { return as_node(Slice(P(x), offsets, sizes)); });
   m.def("Permute", [P](In x, const Shape& s) { return as_node(Permute(P(x), s)); });
   m.def("Transpose", [P](In x, Size i, Size j) { return as_node(Transpose(P(x), i, j)); });
   m.def("RowBroadcast", [P](In x, Size rows) { return as_node(RowBroadcast(P(x), rows)); });
   m.def("ColBroadcast", [P](In x, Size cols) { return as_node(ColBroadcast(P(x), cols)); });
-  m.def("Cat", [](const std::vector<SP<N>>& ins) { return as_node(Cat(ptrs<S>(ins))); });
-  m.def("RowwiseCat", [](const std::vector<SP<N>>& ins) { return as_node(RowwiseCat(ptrs<S>(ins))); });
-  m.def("Stack", [](const std::vector<std::vector<SP<N>>>& grid) {
-    std::vector<std::vector<NodePtr<S>>> g;
-    for (auto& row : grid) g.push_back(ptrs<S>(row));
-    return as_node(Stack<S>(g));
-  });
   m.def("Mask", [P](In x, In mask, double val) { return as_node(Mask(P(x), P(mask), val)); });
   m.def("Select", [P](const SP<Node<bool>>& c, In a, In b) { return as_node(Select(NodePtr<bool>(c), P(a), P(b))); });
-  m.def("LessThan", [P](In a, In b) { return SP<Node<bool>>(LessThan(P(a), P(b)).as_shared_ptr()); });
   auto index_of = [](const SP<DataNode<Int>>& i) { return DataPtr<Int>(i); };
   m.def("Pick", [P, index_of](In x, const SP<DataNode<Int>>& i) { return as_node(Pick(P(x), index_of(i))); });
   m.def("Pick", [P](In x, const std::vector<Int>& i) { return as_node(Pick(P(x), i)); });
@@ -321,11 +331,11 @@ void bind_operators(py::class_<Node<S>, BaseNode, SP<Node<S>>>& c) {
       .def("__sub__", [P](In a, In b) { return as_node(Subtract(P(a), P(b))); })
       .def("__sub__", [P](In a, double s) { return as_node(AddScalar(P(a), -s)); })
       .def("__rsub__", [P](In a, double s) { return as_node(SubtractScalar(s, P(a))); })
-      .def("__mul__", [P](In a, In b) { return as_node(Prod(P(a), P(b))); })
       .def("__mul__", [P](In a, double s) { return as_node(ProdScalar(P(a), s)); })
       .def("__rmul__", [P](In a, double s) { return as_node(ProdScalar(P(a), s)); })
       .def("__neg__", [P](In a) { return as_node(ProdScalar(P(a), -1.)); })
       .def("__lt__", [P](In a, In b) { return SP<Node<bool>>(LessThan(P(a), P(b)).as_shared_ptr()); });
+  if constexpr (is_floating_point_v<S>) c.def("__mul__", [P](In a, In b) { return as_node(Prod(P(a), P(b))); });
 }
 
 // f<S>(args...) for the floating scalar named by `s`, as a Python object.
@@ -408,6 +418,8 @@ PYBIND11_MODULE(ginn, m) {
     bind_operators<Real>(real);
     bind_operators<Half>(half);
     bind_operators<BFloat16>(bf);
+    auto integer = py::class_<Node<Int>, BaseNode, SP<Node<Int>>>(m.attr("IntNode"));
+    bind_operators<Int>(integer);
   }
   // A Real data node converts to every scalar: Values(...).cast(ginn.Half) (ginn/node/data.h:100-108).
   py::class_<DataNode<Real>, Node<Real>, SP<DataNode<Real>>>(m.attr("RealDataNode"))
@@ -464,6 +476,7 @@ PYBIND11_MODULE(ginn, m) {
   bind_float_nodes<Real>(m);
   bind_float_nodes<Half>(m);
   bind_float_nodes<BFloat16>(m);
+  bind_shared_nodes<Int>(m);
 
   // ---- graphs ----
   py::class_<Graph>(m, "Graph")

@@ -43,8 +43,10 @@ typedef enum ginn_hip_dtype {
   GINN_HIP_F32 = 0,
   GINN_HIP_F16 = 1,
   GINN_HIP_BF16 = 2,
-  /* ginn::Int index tensors: accepted only where a declaration says so
-   * (comparison); no arithmetic entry point takes it. */
+  /* ginn::Int tensors (indices, conditions): accepted only where a declaration
+   * says so -- the comparison, and the forward arithmetic of the nodes the
+   * reference instantiates on Int (ginn_hip_add_n, _cwise_prod, _scale_shift,
+   * _elementwise SUB / MAX, _cwise_prod_add_fwd), exact and wrapping. */
   GINN_HIP_I32 = 3
 } ginn_hip_dtype;
 
@@ -366,18 +368,20 @@ int ginn_hip_copy_2d(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows,
 
 /* dst (+)= src_0 + ... + src_{count-1}, n elements each; AddNode forward
  * and the `grad() += ...` of every backward (ginn/node/common.h:116-139).
- * host_srcs is a HOST array of `count` (1..8) device pointers. */
+ * host_srcs is a HOST array of `count` (1..8) device pointers.  dtype may be
+ * GINN_HIP_I32 (Add on Int, test/nodes.cu.cpp:443-487). */
 int ginn_hip_add_n(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n, int count,
                    const void* const* host_srcs, void* dst, int accumulate);
 
 /* dst (+)= a (*) b elementwise; CwiseProdNode forward / backward
- * (ginn/node/common.h:233-262). */
+ * (ginn/node/common.h:233-262).  dtype may be GINN_HIP_I32. */
 int ginn_hip_cwise_prod(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
                         const void* a, const void* b, void* dst,
                         int accumulate);
 
 /* dst (+)= alpha * x + shift; ProdScalar / AddScalar and their backward
- * (ginn/node/common.h:32-95,187-231). */
+ * (ginn/node/common.h:32-95,187-231).  dtype may be GINN_HIP_I32: alpha and
+ * shift are then truncated to integers (the node holds them as Int). */
 int ginn_hip_scale_shift(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
                          float alpha, float shift, const void* x, void* dst,
                          int accumulate);
@@ -470,7 +474,8 @@ int ginn_hip_layernorm_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int rows,
 
 /* CwiseProdAddNode (ginn/node/common.h:251-296): y = a * (b + multiplier_bias)
  * + c.  With broadcast != 0, b and c are [rows] vectors applied to every
- * column of a [rows x cols] (the LayerNorm gamma / beta form). */
+ * column of a [rows x cols] (the LayerNorm gamma / beta form).  dtype may be
+ * GINN_HIP_I32 (forward only). */
 int ginn_hip_cwise_prod_add_fwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
                                 int rows, int cols, const void* a,
                                 const void* b, const void* c,
@@ -580,7 +585,7 @@ typedef enum {
 } ginn_hip_ew_op;
 
 /* dst (+)= op(a, b, c) over n elements; c is read by the three-operand forms
- * only.  dst may be one of the operands. */
+ * only.  dst may be one of the operands.  SUB and MAX also take GINN_HIP_I32. */
 int ginn_hip_elementwise(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
                          ginn_hip_ew_op op, size_t n, const void* a,
                          const void* b, const void* c, void* dst,

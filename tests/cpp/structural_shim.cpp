@@ -452,6 +452,46 @@ void layout_goldens() {
 
 }  // namespace
 
+// Arithmetic nodes with the known answers of test/nodes.cu.cpp:443-640 ("Add subtract": Add, AddScalar,
+// Subtract, SubtractScalar, unary minus, ProdScalar, CwiseProd, CwiseProdAdd with and without a multiplier
+// bias and broadcast operands, CwiseMax), forward, for the floating scalars and for Int.
+template <typename Scalar>
+void arithmetic_goldens() {
+  using N = NodePtr<Scalar>;
+  auto a = on_gpu<Scalar>(Values<2>({{1, 4}, {2, 5}, {3, 6}}));
+  auto b = on_gpu<Scalar>(Values<2>({{-1, 4}, {-2, 5}, {-3, 6}}));
+  auto c = on_gpu<Scalar>(Values<2>({{1, -4}, {2, -5}, {3, -6}}));
+  const Shape s{3, 2};
+  EXPECT_VALUES(Add(N(a), N(b)), s, {0, 0, 0, 8, 10, 12});
+  EXPECT_VALUES(N(a) + N(b), s, {0, 0, 0, 8, 10, 12});
+  EXPECT_VALUES(Add(N(a), N(b), N(c)), s, {1, 2, 3, 4, 5, 6});
+  EXPECT_VALUES(N(a) + N(b) + N(c), s, {1, 2, 3, 4, 5, 6});
+  EXPECT_VALUES(Add(N(a), N(b), N(a)), s, {1, 2, 3, 12, 15, 18});
+  EXPECT_VALUES(AddScalar(a, 1), s, {2, 3, 4, 5, 6, 7});
+  EXPECT_VALUES(a + 1, s, {2, 3, 4, 5, 6, 7});
+  EXPECT_VALUES(1 + a, s, {2, 3, 4, 5, 6, 7});
+  EXPECT_VALUES(Subtract(N(a), N(b)), s, {2, 4, 6, 0, 0, 0});
+  EXPECT_VALUES(N(a) - N(b), s, {2, 4, 6, 0, 0, 0});
+  EXPECT_VALUES(SubtractScalar(1, a), s, {0, -1, -2, -3, -4, -5});
+  EXPECT_VALUES(1 - a, s, {0, -1, -2, -3, -4, -5});
+  EXPECT_VALUES(1.0 - a, s, {0, -1, -2, -3, -4, -5});
+  EXPECT_VALUES(AddScalar(a, -1), s, {0, 1, 2, 3, 4, 5});
+  EXPECT_VALUES(a - 1, s, {0, 1, 2, 3, 4, 5});
+  EXPECT_VALUES(-a, s, {-1, -2, -3, -4, -5, -6});
+  EXPECT_VALUES(ProdScalar(a, 2), s, {2, 4, 6, 8, 10, 12});
+  EXPECT_VALUES(a * 2, s, {2, 4, 6, 8, 10, 12});
+  EXPECT_VALUES(2 * a, s, {2, 4, 6, 8, 10, 12});
+  EXPECT_VALUES(CwiseProd(N(a), N(b)), s, {-1, -4, -9, 16, 25, 36});
+  EXPECT_VALUES(CwiseProdAdd(N(a), N(b), N(c)), s, {0, -2, -6, 12, 20, 30});
+  EXPECT_VALUES(CwiseProdAdd(N(a), N(b), N(c), Scalar(1)), s, {1, 0, -3, 16, 25, 36});  // a (b + 1) + c
+  auto bv = on_gpu<Scalar>(Values<1>({-1, -2, -3}));
+  auto cv = on_gpu<Scalar>(Values<1>({4, 5, 6}));
+  EXPECT_VALUES(CwiseProdAdd(N(a), N(bv), N(cv)), s, {3, 1, -3, 0, -5, -12});
+  EXPECT_VALUES(CwiseProdAdd(N(a), N(bv), N(cv), Scalar(1)), s, {4, 3, 0, 4, 0, -6});
+  EXPECT_VALUES(CwiseMax(N(a), N(b), N(c)), s, {1, 2, 3, 4, 5, 6});
+  EXPECT_VALUES(CwiseMax(N(b), N(c)), s, {1, 2, 3, 4, 5, 6});
+}
+
 extern "C" {
 
 // Runs the named group of checks; returns the report of failed checks ("" = all passed).
@@ -489,6 +529,11 @@ const char* shim_structural(const char* which) {
       layout_goldens<Half>();
       layout_goldens<BFloat16>();
       layout_goldens<Int>();
+    } else if (w == "arithmetic_goldens") {
+      arithmetic_goldens<Real>();
+      arithmetic_goldens<Half>();
+      arithmetic_goldens<BFloat16>();
+      arithmetic_goldens<Int>();
     } else if (w == "arena_limits") {
       arena_limits();
     } else {

@@ -197,7 +197,8 @@ def test_nonlin_nodes(shim, dt, act):
 
 
 @pytest.mark.parametrize("case", ["tensor_ctors", "tensor_ops", "forwardedness", "gradfulness", "arena_tensors",
-                                  "arena_nodes", "arena_limits", "layout_goldens"])
+                                  "arena_nodes", "arena_limits", "layout_goldens",
+                                  "arithmetic_goldens"])
 def test_reference_structural_cases(shim, case):
     """The reference's structural tests on the HIP device: Tensor construction /
     copy / move / assignment across devices, resize, set, serialize and errors
@@ -205,7 +206,8 @@ def test_reference_structural_cases(shim, case):
     (test/graph.cpp:26-115), the byte accounting of the preallocated device
     arena for tensors and nodes (test/dev.cu.cpp:122-178), and the known answers of
     the layout nodes (Stack, Cat, RowwiseCat / RowwiseUncat, Reshape, RankView, Slice,
-    Chip: test/nodes.cu.cpp:66-306) for Real, Half, BFloat16 and Int."""
+    Chip: test/nodes.cu.cpp:66-306) and of the arithmetic nodes (test/nodes.cu.cpp:443-656), both for Real, Half,
+    BFloat16 and Int."""
     shim.shim_structural.restype = ctypes.c_char_p
     report = shim.shim_structural(case.encode()).decode()
     assert report == "", report

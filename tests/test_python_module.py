@@ -246,6 +246,64 @@ def test_reference_python_cases(ginn, scalar_name):
 
 
 @pytest.mark.gpu
+def test_int_nodes_through_the_bindings(ginn):
+    """The cases of ginn-py/test/test_nodes.py that run on ginn.Int (scalars3: Stack :73-118, test_add :388,
+    test_add_scalar :416, test_subtract_scalar :434, test_prod_scalar :459, test_cwise_prod :476, CwiseProdAdd
+    :490-545, test_cwise_max :547, test_reduce :793), on the device, with their known answers; integer
+    arithmetic is exact, so values are compared for equality."""
+    dev = ginn.gpu()
+    I = ginn.Int
+
+    def vals(v):
+        return ginn.Values(dev, v).cast(I)
+
+    def check(node, want):
+        ginn.Graph(node).forward()
+        got = node.value.maybe_copy_to(ginn.cpu())
+        w = vals(want).value.maybe_copy_to(ginn.cpu())
+        assert node.value.scalar == I
+        assert got.shape == w.shape
+        assert got.list() == w.list()
+
+    a = vals([[1, 4], [2, 5], [3, 6]])
+    b = vals([[-1, 4], [-2, 5], [-3, 6]])
+    c = vals([[1, -4], [2, -5], [3, -6]])
+    check(ginn.Add(a, b), [[0, 8], [0, 10], [0, 12]])
+    check(a + b, [[0, 8], [0, 10], [0, 12]])
+    check(ginn.Add([a, b, c]), [[1, 4], [2, 5], [3, 6]])
+    check(a + b + a, [[1, 12], [2, 15], [3, 18]])
+    check(ginn.AddScalar(a, 1), [[2, 5], [3, 6], [4, 7]])
+    check(a + 1, [[2, 5], [3, 6], [4, 7]])
+    check(1 + a, [[2, 5], [3, 6], [4, 7]])
+    check(ginn.Subtract(a, b), [[2, 0], [4, 0], [6, 0]])
+    check(ginn.SubtractScalar(1, a), [[0, -3], [-1, -4], [-2, -5]])
+    check(1 - a, [[0, -3], [-1, -4], [-2, -5]])
+    check(a - 1, [[0, 3], [1, 4], [2, 5]])
+    check(-a, [[-1, -4], [-2, -5], [-3, -6]])
+    check(ginn.ProdScalar(a, 2), [[2, 8], [4, 10], [6, 12]])
+    check(2 * a, [[2, 8], [4, 10], [6, 12]])
+    check(ginn.CwiseProd(a, b), [[-1, 16], [-4, 25], [-9, 36]])
+    check(ginn.CwiseProdAdd(a, b, c), [[0, 12], [-2, 20], [-6, 30]])
+    check(ginn.CwiseProdAdd(a, b, c, 1), [[1, 16], [0, 25], [-3, 36]])
+    bv, cv = vals([-1, -2, -3]), vals([4, 5, 6])
+    check(ginn.CwiseProdAdd(a, bv, cv), [[3, 0], [1, -5], [-3, -12]])
+    check(ginn.CwiseProdAdd(a, bv, cv, 1), [[4, 4], [3, 0], [0, -6]])
+    check(ginn.CwiseMax([b, c]), [[1, 4], [2, 5], [3, 6]])
+    # Stack of rank-1 nodes
+    parts = [vals([1 + 4 * i, 2 + 4 * i, 3 + 4 * i, 4 + 4 * i]) for i in range(6)]
+    check(ginn.Stack([parts[0:2], parts[2:4], parts[4:6]]),
+          [[[1, 5], [9, 13], [17, 21]], [[2, 6], [10, 14], [18, 22]], [[3, 7], [11, 15], [19, 23]],
+           [[4, 8], [12, 16], [20, 24]]])
+    check(ginn.RankView(a, 1), [1, 2, 3, 4, 5, 6])
+    check(ginn.Reshape(a, [2, 3]), [[1, 3, 5], [2, 4, 6]])
+    # comparison
+    x, y = vals([[1], [2], [3], [4], [5]]), vals([[5], [4], [3], [2], [1]])
+    lt = x < y
+    ginn.Graph(lt).forward()
+    assert lt.value.list() == [True, True, False, False, False]
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("scalar_name", ["Half", "BFloat16"])
 def test_mnist_style_training_loop_16bit(ginn, scalar_name):
     """The loop of ginn-py/examples/mnist.py:62-92 with 16-bit weights and
