@@ -171,20 +171,23 @@ def _xavier(rng, rows, cols):
     return rng.uniform(-a, a, (rows, cols))
 
 
-def bench_mlp(iters, cpu, executor=6):
-    """MLP of AffineNodes, fp32, batch 64, 784 -> 512 tanh -> 512 relu -> 10, Sum(PickNegLogSoftmax).
-    executor: 0 = Graph (node by node), 2 = level executor, 6 = level executor frozen after its first pass,
-    14 = the frozen pass recorded as a device graph."""
+def _mlp_case():
+    """Inputs of the MLP configuration: fp32, batch 64, 784 -> 512 tanh -> 512 relu -> 10."""
     import numpy as np
     from ginn_amd import capi
-    ex = _examples()
-    ex.scenario_set_executor(executor)
     rng = np.random.default_rng(1)
     dims, acts, batch = [784, 512, 512, 10], [capi.ACT_TANH, capi.ACT_RELU, capi.ACT_IDENTITY], 64
     x = _f32(rng.uniform(0, 1, (dims[0], batch)))
     labels = rng.integers(0, 10, batch).astype(np.int32)
     Ws = [_f32(_xavier(rng, dims[i + 1], dims[i])) for i in range(3)]
     bs = [_f32(_xavier(rng, dims[i + 1], 1).reshape(-1)) for i in range(3)]
+    return dims, acts, batch, x, labels, Ws, bs
+
+
+def _run_mlp(ex, iters, case):
+    """scenario_mlp on `case`: (ms per pass, loss, per-example losses, dW, db)."""
+    import numpy as np
+    dims, acts, batch, x, labels, Ws, bs = case
     dWs, dbs = [np.zeros_like(w) for w in Ws], [np.zeros_like(b) for b in bs]
     loss, nll, ms = np.zeros(1, np.float32), np.zeros(batch, np.float32), ctypes.c_float(0)
     rc = ex.scenario_mlp(0, batch, 3, (ctypes.c_int * 4)(*dims), (ctypes.c_int * 3)(*acts), _fp(x),
@@ -193,6 +196,31 @@ def bench_mlp(iters, cpu, executor=6):
                          (FP * 3)(*map(_fp, dbs)), ctypes.byref(ms))
     if rc:
         raise SystemExit(ex.scenario_last_error().decode())
+    return ms.value, loss, nll, dWs, dbs
+
+
+def mlp_on_host_nodes(iters):
+    """The MLP configuration forward + backward with its graph on cpu(): the same example graph as on the
+    device, run node by node through the host layer's own loops (ginn_amd/ginn/cpu_ops.h, one thread).
+    Returns (ms per pass, loss, per-example losses, dW, db); touches no GPU."""
+    ex = _examples()
+    ex.scenario_set_executor(0)
+    ex.scenario_set_device(1)
+    try:
+        return _run_mlp(ex, iters, _mlp_case())
+    finally:
+        ex.scenario_set_device(0)
+
+
+def bench_mlp(iters, cpu, executor=6):
+    """MLP of AffineNodes, fp32, batch 64, 784 -> 512 tanh -> 512 relu -> 10, Sum(PickNegLogSoftmax).
+    executor: 0 = Graph (node by node), 2 = level executor, 6 = level executor frozen after its first pass,
+    14 = the frozen pass recorded as a device graph."""
+    ex = _examples()
+    ex.scenario_set_executor(executor)
+    case = _mlp_case()
+    dims, acts, batch, x, labels, Ws, bs = case
+    ms = _run_mlp(ex, iters, case)[0]
     flops = 3 * sum(2.0 * dims[i + 1] * dims[i] * batch for i in range(3)) - 2.0 * 512 * 784 * batch
     ex.scenario_set_executor(0)
     # Algorithmic bytes of the pass: 4 (M K + K N + M N (1 + beta)) over its eight products (three forward,
@@ -202,14 +230,16 @@ def bench_mlp(iters, cpu, executor=6):
         mm, kk = dims[i + 1], dims[i]
         per = 4.0 * (mm * kk + kk * batch + mm * batch)
         by += per * (3 if i else 2)
-    r = {"config": f"mlp fp32 b64 784-512-512-10 fwd+bwd, executor={executor}", "gpu_ms": round(ms.value, 4),
-         "gflops": round(flops / ms.value / 1e6, 1), "gbs": round(by / ms.value / 1e6, 1), "algorithmic_bytes": int(by)}
+    r = {"config": f"mlp fp32 b64 784-512-512-10 fwd+bwd, executor={executor}", "gpu_ms": round(ms, 4),
+         "gflops": round(flops / ms / 1e6, 1), "gbs": round(by / ms / 1e6, 1), "algorithmic_bytes": int(by)}
     if executor & 8:
         r["kernels_per_pass"] = int(ex.scenario_recorded_kernels())
     if cpu:
         from oracle import nodes as N
         r["cpu_ms"] = round(_cpu_timed(lambda: N.mlp_forward_backward(acts, Ws, bs, x, labels)), 3)
         r["cpu"] = "oracle (numpy fp32 restatement), 1 thread"
+        r["cpu_nodes_ms"] = round(mlp_on_host_nodes(10)[0], 3)
+        r["cpu_nodes"] = "the same graph on cpu(): host layer nodes over their own fp32 loops, 1 thread"
     return r
 
 
@@ -526,6 +556,7 @@ def other_configs(h, cpu):
     out["mlp_ms"], out["mlp_gbs"] = r["gpu_ms"], r["gbs"]
     if cpu:
         out["mlp_cpu_ms"] = r["cpu_ms"]
+        out["mlp_cpu_nodes_ms"] = r["cpu_nodes_ms"]
     out["mlp_kernels_per_pass"] = bench_mlp(2, False, executor=14)["kernels_per_pass"]
     r = bench_lstm(10, cpu, mode=23, gather=True)
     out["lstm_ms"], out["lstm_gbs"] = r["gpu_ms"], r["gbs"]
@@ -555,7 +586,8 @@ def other_configs(h, cpu):
                    "autobatched LSTM fp32 256 seqs; gbs = algorithmic bytes of the pass's products per second; "
                    "kernels_per_pass = kernel nodes of the pass recorded as a device graph; attention = fp16 batch 128 "
                    "products, skinny = M = K = 4096 NN with the split-K fold included, against 8 TB/s; squares "
-                   "against 2.5 PFLOP/s; cpu = numpy fp32 oracle on 1 thread")
+                   "against 2.5 PFLOP/s; cpu = numpy fp32 oracle on 1 thread; mlp_cpu_nodes_ms = the same MLP graph with "
+                   "its nodes on cpu() (the host layer's own fp32 loops, 1 thread)")
     return out
 
 

@@ -27,6 +27,10 @@ using namespace ginn;
 namespace {
 
 thread_local std::string g_error;
+// scenario_set_device(1): the MLP scenario keeps its graph on cpu() and runs through the host layer's own
+// loops (ginn/cpu_ops.h), node by node -- the same graph code as on the device, as a host baseline.
+bool g_on_cpu = false;
+DevPtr place() { return g_on_cpu ? DevPtr(cpu()) : DevPtr(gpu()); }
 
 template <typename S>
 void upload(Tensor<S>& t, const float* vals) {
@@ -45,7 +49,7 @@ void read_back(const Tensor<S>& t, float* out) {
 
 template <typename S>
 Ptr<DataNode<S>> data_from(const Shape& shape, const float* vals, bool has_grad) {
-  auto x = Data<S>(gpu(), shape);
+  auto x = Data<S>(place(), shape);
   upload(x->value(), vals);
   x->set_has_grad(has_grad);
   return x;
@@ -53,7 +57,7 @@ Ptr<DataNode<S>> data_from(const Shape& shape, const float* vals, bool has_grad)
 
 template <typename S>
 Ptr<WeightNode<S>> weight_from(const Shape& shape, const float* vals) {
-  auto w = Weight<S>(gpu(), shape);
+  auto w = Weight<S>(place(), shape);
   upload(w->value(), vals);
   return w;
 }
@@ -93,7 +97,7 @@ std::unique_ptr<Updater<S>> make_updater() {
 // One training-style pass, `iters` times: forward, reset_grad, backward(1).
 // Returns the mean wall time per pass (device drained on both sides).
 double run_passes(Graph& g, int iters) {
-  gpu()->synchronize();
+  if (!g_on_cpu) gpu()->synchronize();
   const double t0 = now_ms();
   for (int it = 0; it < iters; ++it) {
     g.reset_forwarded();
@@ -102,7 +106,7 @@ double run_passes(Graph& g, int iters) {
     g.backward(1.);
     if (g_after_backward) g_after_backward();
   }
-  gpu()->synchronize();
+  if (!g_on_cpu) gpu()->synchronize();
   return (now_ms() - t0) / (iters > 0 ? iters : 1);
 }
 
@@ -156,7 +160,7 @@ struct FillCount {
 // Warm-up pass (first-touch allocations, launch plans), then `iters` timed ones.
 double run_warm(Graph& g, int iters) {
   FillCount count;
-  if (g_exec_mode & 2) {
+  if ((g_exec_mode & 2) && !g_on_cpu) {
     LevelExecutor ex(g);
     run_passes(ex, 1);
     if (g_exec_mode & 4) ex.freeze();
@@ -183,7 +187,7 @@ int mlp(int batch, int n_layers, const int* dims, const int* acts, const float* 
   auto X = data_from<S>({dims[0], batch}, x, false);
   auto Y = Data<Int>(cpu(), Shape{batch});
   for (int i = 0; i < batch; ++i) Y->value().v()[i] = labels[i];
-  Y->move_to(gpu());
+  Y->move_to(place());
   Y->set_has_grad(false);
 
   std::vector<Ptr<WeightNode<S>>> Ws, bs;
@@ -599,6 +603,8 @@ int scenario_lstm(int mode, int nseq, const int* lens, int E, int H, const float
 // node), 2 = level executor, 6 = level executor frozen after its first pass, 14 = the frozen pass as a
 // recorded device graph.
 void scenario_set_executor(int mode) { g_exec_mode = mode; }
+// 1: scenario_mlp builds and runs its graph on cpu() (host loops, node by node); 0: on the HIP device.
+void scenario_set_device(int on_cpu) { g_on_cpu = on_cpu != 0; }
 
 // Training rule of scenario_gpt_layer from now on: -1 = none (forward + backward only), 0 = Sgd, 1 = Adam;
 // every pass then ends with updater.update(all weights).  out_loss is the loss of the last pass.

@@ -1,0 +1,252 @@
+// The host layer's own arithmetic for tensors on cpu(): plain loops with fp32
+// accumulation behind the nodes of the product path (Prod, BatchedProd,
+// Affine, the nonlinearities, Add / Subtract / CwiseProd / the scalar forms,
+// Sum / Mean, PickNegLogSoftmax), so that the same graph code runs on either
+// device as in the reference (ginn/node/prod.h:31-46, ginn/node/affine.h:49-53,
+// ginn/nonlin.h:67-300, where the CPU side is Eigen expressions).  A reference
+// point for the device path, single-threaded like the reference's Eigen build;
+// nothing here is called for a tensor on the HIP device.
+#ifndef GINN_CPU_OPS_H
+#define GINN_CPU_OPS_H
+
+#include <algorithm>
+#include <cmath>
+#include <cstddef>
+#include <type_traits>
+#include <vector>
+
+#include <ginn/def.h>
+
+namespace ginn {
+namespace host {
+
+template <typename S>
+inline float get(const S* p, size_t i) {
+  return static_cast<float>(p[i]);
+}
+template <typename S>
+inline void put(S* p, size_t i, float v) {
+  p[i] = S(v);
+}
+
+// An operand as fp32, column-major with leading dimension ld: the tensor's own
+// memory for Real, a converted copy (kept in `keep`) for the 16-bit types.
+template <typename S>
+inline const float* as_f32(const S* src, size_t ld, size_t cols, std::vector<float>& keep) {
+  if constexpr (std::is_same_v<S, float>) {
+    return src;
+  } else {
+    keep.resize(ld * cols);
+    for (size_t i = 0; i < ld * cols; ++i) keep[i] = static_cast<float>(src[i]);
+    return keep.data();
+  }
+}
+
+// C[m x n] = op(A)[m x k] * op(B)[k x n] + beta * C, column-major, fp32 accumulation, one rounding to S.
+// Blocked over K (the panel of A a column block of C reuses stays in cache) with four columns of C per sweep
+// over a column of A; a transposed A turns the sweep into dot products of contiguous columns.
+template <typename S>
+void gemm(bool ta, bool tb, int m, int n, int k, const S* A, int lda, const S* B, int ldb, float beta, S* C,
+          int ldc) {
+  if (m <= 0 || n <= 0) return;
+  std::vector<float> keep_a, keep_b;
+  const float* a = as_f32(A, static_cast<size_t>(lda), static_cast<size_t>(ta ? m : k), keep_a);
+  const float* b = as_f32(B, static_cast<size_t>(ldb), static_cast<size_t>(tb ? k : n), keep_b);
+  auto b_at = [&](int l, int j) { return tb ? b[j + static_cast<size_t>(l) * ldb] : b[l + static_cast<size_t>(j) * ldb]; };
+  std::vector<float> acc(static_cast<size_t>(m) * 4);
+  constexpr int kBlockK = 256;
+  for (int j0 = 0; j0 < n; j0 += 4) {
+    const int nj = std::min(4, n - j0);
+    std::fill(acc.begin(), acc.end(), 0.f);
+    float* c0 = acc.data();
+    float* c1 = c0 + m;
+    float* c2 = c1 + m;
+    float* c3 = c2 + m;
+    float* cols[4] = {c0, c1, c2, c3};
+    if (!ta) {
+      for (int l0 = 0; l0 < k; l0 += kBlockK) {
+        const int l1 = std::min(k, l0 + kBlockK);
+        for (int l = l0; l < l1; ++l) {
+          const float* al = a + static_cast<size_t>(l) * lda;
+          if (nj == 4) {
+            const float b0 = b_at(l, j0), b1 = b_at(l, j0 + 1), b2 = b_at(l, j0 + 2), b3 = b_at(l, j0 + 3);
+            for (int i = 0; i < m; ++i) {
+              const float v = al[i];
+              c0[i] += v * b0;
+              c1[i] += v * b1;
+              c2[i] += v * b2;
+              c3[i] += v * b3;
+            }
+          } else {
+            for (int jj = 0; jj < nj; ++jj) {
+              const float bv = b_at(l, j0 + jj);
+              float* c = cols[jj];
+              for (int i = 0; i < m; ++i) c[i] += al[i] * bv;
+            }
+          }
+        }
+      }
+    } else {
+      // op(A)(i, l) = A(l, i): column i of the stored A against column j of op(B)
+      std::vector<float> bcol(static_cast<size_t>(k));
+      for (int jj = 0; jj < nj; ++jj) {
+        for (int l = 0; l < k; ++l) bcol[l] = b_at(l, j0 + jj);
+        float* c = cols[jj];
+        for (int i = 0; i < m; ++i) {
+          const float* ai = a + static_cast<size_t>(i) * lda;
+          float s = 0.f;
+          for (int l = 0; l < k; ++l) s += ai[l] * bcol[l];
+          c[i] = s;
+        }
+      }
+    }
+    for (int jj = 0; jj < nj; ++jj) {
+      S* out = C + static_cast<size_t>(j0 + jj) * ldc;
+      const float* c = cols[jj];
+      if (beta != 0.f)
+        for (int i = 0; i < m; ++i) put(out, i, c[i] + beta * get(out, i));
+      else
+        for (int i = 0; i < m; ++i) put(out, i, c[i]);
+    }
+  }
+}
+
+// The nonlinearities (ginn/nonlin.h:67-300) on one value; `code` as in the device library.
+inline float act_forward(int code, float x) {
+  switch (code) {
+    case GINN_HIP_ACT_TANH: return std::tanh(x);
+    case GINN_HIP_ACT_RELU: return x > 0.f ? x : 0.f;
+    case GINN_HIP_ACT_SIGMOID: return 0.5f * std::tanh(0.5f * x) + 0.5f;  // ginn/nonlin.h:141-144
+    case GINN_HIP_ACT_GELU: return 0.5f * x * (1.f + std::erf(x * 0.70710678118654752440f));  // :281-283
+    case GINN_HIP_ACT_GELU2: {  // :250-254
+      const float a = 0.79788456080286535588f, b = 0.044715f;
+      return 0.5f * x * (1.f + std::tanh(a * (x + b * x * x * x)));
+    }
+    case GINN_HIP_ACT_LOG: return std::log(x);
+    case GINN_HIP_ACT_SQRT: return std::sqrt(x);
+    default: return x;
+  }
+}
+// d f(x) / dx from the input x and the output y (each nonlinearity's `backward` there).
+inline float act_derivative(int code, float x, float y) {
+  switch (code) {
+    case GINN_HIP_ACT_TANH: return 1.f - y * y;
+    case GINN_HIP_ACT_RELU: return y > 0.f ? 1.f : 0.f;
+    case GINN_HIP_ACT_SIGMOID: return y * (1.f - y);
+    case GINN_HIP_ACT_GELU:  // :290-296
+      return 0.5f * (1.f + std::erf(x * 0.70710678118654752440f)) +
+             x * std::exp(-0.5f * x * x) * 0.39894228040143267794f;
+    case GINN_HIP_ACT_GELU2: {  // :262-266, written without the division by x
+      const float a = 0.79788456080286535588f, b = 0.044715f;
+      const float t = std::tanh(a * (x + b * x * x * x));
+      return 0.5f * (1.f + t) + 0.5f * x * (1.f - t * t) * a * (1.f + 3.f * b * x * x);
+    }
+    case GINN_HIP_ACT_LOG: return 1.f / x;
+    case GINN_HIP_ACT_SQRT: return 0.5f / y;
+    default: return 1.f;
+  }
+}
+
+// y = f(x) over [rows x cols]; SOFTMAX is taken per column (ginn/nonlin.h:150-175).
+template <typename S>
+void nonlin_forward(int code, int rows, int cols, const S* x, S* y) {
+  if (code == GINN_HIP_ACT_SOFTMAX) {
+    std::vector<float> e(static_cast<size_t>(rows));
+    for (int c = 0; c < cols; ++c) {
+      const S* xc = x + static_cast<size_t>(c) * rows;
+      S* yc = y + static_cast<size_t>(c) * rows;
+      float mx = -INFINITY, sum = 0.f;
+      for (int r = 0; r < rows; ++r) mx = std::max(mx, get(xc, r));
+      for (int r = 0; r < rows; ++r) sum += (e[r] = std::exp(get(xc, r) - mx));
+      for (int r = 0; r < rows; ++r) put(yc, r, e[r] / sum);
+    }
+    return;
+  }
+  const size_t n = static_cast<size_t>(rows) * cols;
+  for (size_t i = 0; i < n; ++i) put(y, i, act_forward(code, get(x, i)));
+}
+// dx (+)= f'(x, y) (*) dy; SOFTMAX: dx = y (*) (dy - <dy, y>) per column (ginn/nonlin.h:177-184).
+template <typename S>
+void nonlin_backward(int code, int rows, int cols, const S* dy, const S* x, const S* y, S* dx, bool accumulate) {
+  if (code == GINN_HIP_ACT_SOFTMAX) {
+    for (int c = 0; c < cols; ++c) {
+      const size_t o = static_cast<size_t>(c) * rows;
+      float dot = 0.f;
+      for (int r = 0; r < rows; ++r) dot += get(dy, o + r) * get(y, o + r);
+      for (int r = 0; r < rows; ++r) {
+        const float v = get(y, o + r) * (get(dy, o + r) - dot);
+        put(dx, o + r, accumulate ? get(dx, o + r) + v : v);
+      }
+    }
+    return;
+  }
+  const size_t n = static_cast<size_t>(rows) * cols;
+  for (size_t i = 0; i < n; ++i) {
+    const float v = get(dy, i) * act_derivative(code, x ? get(x, i) : 0.f, y ? get(y, i) : 0.f);
+    put(dx, i, accumulate ? get(dx, i) + v : v);
+  }
+}
+
+// dst (+)= alpha * x + shift; dst (+)= a (*) b; dst (+)= a + sign * b.
+template <typename S>
+void scale_shift(size_t n, float alpha, float shift, const S* x, S* dst, bool accumulate) {
+  for (size_t i = 0; i < n; ++i) {
+    const float v = alpha * get(x, i) + shift;
+    put(dst, i, accumulate ? get(dst, i) + v : v);
+  }
+}
+template <typename S>
+void cwise_prod(size_t n, const S* a, const S* b, S* dst, bool accumulate) {
+  for (size_t i = 0; i < n; ++i) {
+    const float v = get(a, i) * get(b, i);
+    put(dst, i, accumulate ? get(dst, i) + v : v);
+  }
+}
+template <typename S>
+void add_n(size_t n, const std::vector<const S*>& srcs, S* dst, bool accumulate) {
+  for (size_t i = 0; i < n; ++i) {
+    float v = accumulate ? get(dst, i) : 0.f;
+    for (const S* s : srcs) v += get(s, i);
+    put(dst, i, v);
+  }
+}
+
+// sum of all elements (scale = 1) or their mean (scale = 1 / n), fp32 accumulation.
+template <typename S>
+float sum_all(size_t n, const S* x) {
+  double s = 0.;
+  for (size_t i = 0; i < n; ++i) s += get(x, i);
+  return static_cast<float>(s);
+}
+
+// PickNegLogSoftmax per column (ginn/node/pick.h: -log softmax(x)[index]) and its gradient
+// dx (+)= (softmax(x) - onehot(index)) * dy[c].
+template <typename S>
+void pick_nls_forward(int rows, int cols, const S* x, const int* index, S* out) {
+  for (int c = 0; c < cols; ++c) {
+    const S* xc = x + static_cast<size_t>(c) * rows;
+    float mx = -INFINITY, sum = 0.f;
+    for (int r = 0; r < rows; ++r) mx = std::max(mx, get(xc, r));
+    for (int r = 0; r < rows; ++r) sum += std::exp(get(xc, r) - mx);
+    put(out, c, -(get(xc, index[c]) - mx - std::log(sum)));
+  }
+}
+template <typename S>
+void pick_nls_backward(int rows, int cols, const S* x, const int* index, const S* dy, S* dx, bool accumulate) {
+  for (int c = 0; c < cols; ++c) {
+    const size_t o = static_cast<size_t>(c) * rows;
+    float mx = -INFINITY, sum = 0.f;
+    for (int r = 0; r < rows; ++r) mx = std::max(mx, get(x, o + r));
+    for (int r = 0; r < rows; ++r) sum += std::exp(get(x, o + r) - mx);
+    const float g = get(dy, c);
+    for (int r = 0; r < rows; ++r) {
+      const float v = (std::exp(get(x, o + r) - mx) / sum - (r == index[c] ? 1.f : 0.f)) * g;
+      put(dx, o + r, accumulate ? get(dx, o + r) + v : v);
+    }
+  }
+}
+
+}  // namespace host
+}  // namespace ginn
+
+#endif  // GINN_CPU_OPS_H

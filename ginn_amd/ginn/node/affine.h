@@ -27,7 +27,59 @@ class AffineNode : public BaseDataNode<Scalar> {
     GINN_ASSERT(ins_.size() % 2);  // pairs plus the bias
   }
 
+  // On cpu(): the reference's own sequence (ginn/node/affine.h:35-77) -- bias broadcast, one accumulating
+  // product per pair, the nonlinearity -- in the host layer's loops.
+  void forward_cpu() {
+    auto& bias = ins_.back()->value();
+    Shape out = ins_[1]->value().shape();
+    out[0] = ins_[0]->value().rows();
+    const Size m = out[0];
+    GINN_ASSERT(bias.size() == m, "Affine bias must have one entry per output row!");
+    const bool keep_pre = nonlin_->backward_requires_input();
+    value().resize(out);
+    Tensor<Scalar>& pre = keep_pre ? preactiv_ : value();
+    if (keep_pre) preactiv_.resize(out);
+    const Size n = pre.cols();
+    for (Size c = 0; c < n; ++c)
+      for (Size r = 0; r < m; ++r) pre.data()[c * m + r] = bias.data()[r];
+    for (size_t i = 0; i + 1 < ins_.size(); i += 2) {
+      GINN_ASSERT(ins_[i]->value().shape().size() == 2);
+      internal::cpu_prod(pre, ins_[i]->value(), ins_[i + 1]->value(), internal::ProdResult::Add);
+    }
+    if (!nonlin_->is_identity()) nonlin_->forward(value(), pre);
+  }
+  void backward_cpu() {
+    using namespace internal;
+    const bool identity = nonlin_->is_identity();
+    Tensor<Scalar>& daffine = identity ? grad() : dpreactiv_;
+    if (!identity) {
+      dpreactiv_.resize(grad().shape());
+      nonlin_->backward(dpreactiv_, grad(), preactiv_, value(), false);
+    }
+    auto& bias = ins_.back();
+    const Size m = grad().rows(), n = grad().cols();
+    if (bias->has_grad()) {
+      const bool fresh = bias->take_lazy_zero();
+      Scalar* db = bias->grad().data();
+      for (Size r = 0; r < m; ++r) {
+        float s = fresh ? 0.f : static_cast<float>(db[r]);
+        for (Size c = 0; c < n; ++c) s += static_cast<float>(daffine.data()[c * m + r]);
+        db[r] = Scalar(s);
+      }
+    }
+    for (size_t i = 0; i + 1 < ins_.size(); i += 2) {
+      auto &a = ins_[i], &b = ins_[i + 1];
+      if (b->has_grad())
+        cpu_prod(b->grad(), a->value(), daffine, b->take_lazy_zero() ? ProdResult::Assign : ProdResult::Add,
+                 ProdTranspose::First);
+      if (a->has_grad())
+        cpu_prod(a->grad(), daffine, b->value(), a->take_lazy_zero() ? ProdResult::Assign : ProdResult::Add,
+                 ProdTranspose::Second);
+    }
+  }
+
   void forward_() override {
+    if (dev()->kind() == CPU) return forward_cpu();
     internal::require_gpu(dev(), "Affine");
     auto& a0 = ins_[0]->value();
     auto& b0 = ins_[1]->value();
@@ -65,6 +117,7 @@ class AffineNode : public BaseDataNode<Scalar> {
 
   void backward_() override {
     using namespace internal;
+    if (dev()->kind() == CPU) return backward_cpu();
     const bool identity = nonlin_->is_identity();
     Tensor<Scalar>& daffine = identity ? grad() : dpreactiv_;
     if (!identity) dpreactiv_.resize(grad().shape());

@@ -15,8 +15,18 @@ namespace internal {
 // dst (+)= sum of srcs, in groups of eight per launch.
 template <typename Scalar>
 void add_tensors(Tensor<Scalar>& dst, const std::vector<const Tensor<Scalar>*>& srcs, bool accumulate) {
-  require_gpu(dst.dev(), "Add");
   const size_t n = static_cast<size_t>(dst.size());
+  if (dst.dev()->kind() == CPU) {
+    std::vector<const Scalar*> p;
+    for (auto* s : srcs) {
+      GINN_ASSERT(s->size() == dst.size(), "Add: operand sizes differ");
+      p.push_back(s->data());
+    }
+    if constexpr (is_floating_point_v<Scalar>) host::add_n<Scalar>(n, p, dst.data(), accumulate);
+    else GINN_THROW("Add on cpu(): floating-point scalars only");
+    return;
+  }
+  require_gpu(dst.dev(), "Add");
   for (size_t i = 0; i < srcs.size(); i += 8) {
     const int count = static_cast<int>(std::min<size_t>(8, srcs.size() - i));
     const void* p[8];
@@ -110,6 +120,10 @@ class CwiseProdNode : public BaseDataNode<Scalar> {
   NodePtr<Scalar> a_, b_;
 
   void run(Tensor<Scalar>& dst, const Tensor<Scalar>& x, const Tensor<Scalar>& y, bool acc) {
+    if (dst.dev()->kind() == CPU) {
+      if constexpr (is_floating_point_v<Scalar>)
+        return host::cwise_prod<Scalar>(static_cast<size_t>(dst.size()), x.data(), y.data(), dst.data(), acc);
+    }
     internal::require_gpu(dst.dev(), "CwiseProd");
     GINN_HIP_CALL(ginn_hip_cwise_prod(internal::ctx_of(dst), arith_dtype_of<Scalar>(), static_cast<size_t>(dst.size()),
                                       x.data(), y.data(), dst.data(), acc ? 1 : 0));
@@ -185,8 +199,13 @@ class ScaleShiftNode : public BaseDataNode<Scalar> {
   const char* name_;
 
   void forward_() override {
-    internal::require_gpu(this->dev(), name_);
     value().resize(in_->value().shape());
+    if (this->dev()->kind() == CPU) {
+      if constexpr (is_floating_point_v<Scalar>)
+        return host::scale_shift<Scalar>(static_cast<size_t>(value().size()), alpha_, shift_, in_->value().data(),
+                                        value().data(), false);
+    }
+    internal::require_gpu(this->dev(), name_);
     GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(value()), arith_dtype_of<Scalar>(),
                                        static_cast<size_t>(value().size()), alpha_, shift_, in_->value().data(),
                                        value().data(), 0));
@@ -194,6 +213,11 @@ class ScaleShiftNode : public BaseDataNode<Scalar> {
   void backward_() override {
     if (!in_->has_grad()) return;
     const bool fresh = in_->take_lazy_zero();
+    if (this->dev()->kind() == CPU) {
+      if constexpr (is_floating_point_v<Scalar>)
+        return host::scale_shift<Scalar>(static_cast<size_t>(grad().size()), alpha_, 0.f, grad().data(),
+                                        in_->grad().data(), !fresh);
+    }
     GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(grad()), arith_dtype_of<Scalar>(),
                                        static_cast<size_t>(grad().size()), alpha_, 0.f, grad().data(),
                                        in_->grad().data(), fresh ? 0 : 1));

@@ -104,8 +104,16 @@ class PickNegLogSoftmaxNode : public PickSoftmaxNode<Scalar> {
   Tensor<float> stats_;  // per column: maximum, 1 / sum of exp(x - maximum)
 
   void forward_() override {
-    internal::require_gpu(this->dev(), "PickNegLogSoftmax");
     auto& x = in_->value();
+    if (this->dev()->kind() == CPU) {  // the host layer's loops (ginn/cpu_ops.h)
+      GINN_ASSERT(x.cols() == index_->value().size(), "Index size does not match input columns!");
+      GINN_ASSERT(index_->dev()->kind() == CPU, "PickNegLogSoftmax: index and input must live on one device");
+      value().resize(1, x.cols());
+      host::pick_nls_forward<Scalar>(static_cast<int>(x.rows()), static_cast<int>(x.cols()), x.data(),
+                                    index_->value().data(), value().data());
+      return;
+    }
+    internal::require_gpu(this->dev(), "PickNegLogSoftmax");
     this->check_index(x);
     stats_.move_to(this->dev());
     stats_.resize(2, x.cols());
@@ -118,6 +126,11 @@ class PickNegLogSoftmaxNode : public PickSoftmaxNode<Scalar> {
     if (!in_->has_grad()) return;
     auto& x = in_->value();
     const bool fresh = in_->take_lazy_zero();
+    if (this->dev()->kind() == CPU) {
+      host::pick_nls_backward<Scalar>(static_cast<int>(x.rows()), static_cast<int>(x.cols()), x.data(),
+                                     index_->value().data(), grad().data(), in_->grad().data(), !fresh);
+      return;
+    }
     GINN_HIP_CALL(ginn_hip_pick_nls_bwd_stats(internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()),
                                               static_cast<int>(x.cols()), x.data(), stats_.data(),
                                               index_->value().data(), grad().data(), in_->grad().data(),

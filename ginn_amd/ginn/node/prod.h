@@ -18,12 +18,25 @@ class ProdNode : public BaseDataNode<Scalar> {
   NodePtr<Scalar> a_, b_;
 
   void forward_() override {
-    internal::require_gpu(dev(), "Prod");
     value().resize(a_->value().rows(), b_->value().cols());
+    if (dev()->kind() == CPU) {
+      internal::cpu_prod(value(), a_->value(), b_->value());
+      return;
+    }
+    internal::require_gpu(dev(), "Prod");
     internal::gpu_prod(value(), a_->value(), b_->value());
   }
   void backward_() override {
     using namespace internal;
+    if (dev()->kind() == CPU) {  // ginn/node/prod.h:39-58
+      if (b_->has_grad())
+        cpu_prod(b_->grad(), a_->value(), grad(), b_->take_lazy_zero() ? ProdResult::Assign : ProdResult::Add,
+                 ProdTranspose::First);
+      if (a_->has_grad())
+        cpu_prod(a_->grad(), grad(), b_->value(), a_->take_lazy_zero() ? ProdResult::Assign : ProdResult::Add,
+                 ProdTranspose::Second);
+      return;
+    }
     // A gradient that is a leaf's (a weight's) is formed beside the pass, the other one first.
     const double flops = 2.0 * static_cast<double>(grad().size()) * static_cast<double>(a_->value().cols());
     for (const bool leaves : {false, true}) {
@@ -326,14 +339,27 @@ class BatchedProdNode : public BaseDataNode<Scalar> {
     GINN_ASSERT(sa.size() == sb.size(), "Mismatching batch dimensions in BatchedProd!");
     for (size_t i = 2; i < sa.size(); ++i)
       GINN_ASSERT(sa[i] == sb[i], "Mismatching batch dimensions in BatchedProd!");
-    internal::require_gpu(dev(), "BatchedProd");
     Shape s = sb;
     s[0] = sa[0];
     value().resize(s);
+    if (dev()->kind() == CPU) {
+      internal::cpu_batched_prod(value(), a_->value(), b_->value());
+      return;
+    }
+    internal::require_gpu(dev(), "BatchedProd");
     internal::gpu_batched_prod(value(), a_->value(), b_->value());
   }
   void backward_() override {
     using namespace internal;
+    if (dev()->kind() == CPU) {
+      if (a_->has_grad())
+        cpu_batched_prod(a_->grad(), grad(), b_->value(),
+                         a_->take_lazy_zero() ? ProdResult::Assign : ProdResult::Add, ProdTranspose::Second);
+      if (b_->has_grad())
+        cpu_batched_prod(b_->grad(), a_->value(), grad(),
+                         b_->take_lazy_zero() ? ProdResult::Assign : ProdResult::Add, ProdTranspose::First);
+      return;
+    }
     if (a_->has_grad()) {
       const bool fresh = a_->take_lazy_zero();
       gpu_batched_prod(a_->grad(), grad(), b_->value(), fresh ? ProdResult::Assign : ProdResult::Add,

@@ -17,13 +17,24 @@ class SumNode : public BaseDataNode<Scalar> {
   virtual float scale() const { return 1.f; }
 
   void forward_() override {
-    internal::require_gpu(this->dev(), name().c_str());
     value().resize({});
+    if (this->dev()->kind() == CPU) {
+      value().data()[0] = Scalar(scale() * host::sum_all<Scalar>(static_cast<size_t>(in_->value().size()),
+                                                                 in_->value().data()));
+      return;
+    }
+    internal::require_gpu(this->dev(), name().c_str());
     GINN_HIP_CALL(ginn_hip_sum_all(internal::ctx_of(value()), dtype_of<Scalar>(),
                                    static_cast<size_t>(in_->value().size()), in_->value().data(), scale(),
                                    value().data()));
   }
   void backward_() override {
+    if (in_->has_grad() && this->dev()->kind() == CPU) {
+      const float g = scale() * static_cast<float>(grad().data()[0]);
+      Scalar* dx = in_->grad().data();
+      for (Size i = 0; i < in_->grad().size(); ++i) dx[i] = Scalar(static_cast<float>(dx[i]) + g);
+      return;
+    }
     if (in_->has_grad())
       GINN_HIP_CALL(ginn_hip_add_scalar_bcast(internal::ctx_of(grad()), dtype_of<Scalar>(),
                                               static_cast<size_t>(in_->grad().size()), grad().data(), scale(),

@@ -13,7 +13,7 @@ namespace ginn {
 
 namespace internal {
 inline void require_gpu(const DevPtr& dev, const char* what) {
-  GINN_ASSERT(dev->kind() == GPU, std::string(what) + ": this build computes on the HIP device only "
+  GINN_ASSERT(dev->kind() == GPU, std::string(what) + ": this node computes on the HIP device only "
                                                       "(move the inputs with move_to(gpu()))");
 }
 template <typename Scalar>
@@ -31,8 +31,12 @@ class NonlinOp {
   virtual bool is_identity() const { return false; }
 
   virtual void forward(Tensor<Scalar>& y, const Tensor<Scalar>& x) const {
-    internal::require_gpu(x.dev(), "NonlinOp::forward");
     y.resize(x.shape());
+    if (x.dev()->kind() == CPU) {  // ginn/nonlin.h:67-300 on the host
+      host::nonlin_forward<Scalar>(code(), static_cast<int>(x.rows()), static_cast<int>(x.cols()), x.data(), y.data());
+      return;
+    }
+    internal::require_gpu(x.dev(), "NonlinOp::forward");
     GINN_HIP_CALL(ginn_hip_nonlin_fwd(internal::ctx_of(x), dtype_of<Scalar>(), code(),
                                       static_cast<int>(x.rows()), static_cast<int>(x.cols()), x.data(),
                                       y.data()));
@@ -40,6 +44,12 @@ class NonlinOp {
   // x may be an empty tensor when backward_requires_input() is false.
   virtual void backward(Tensor<Scalar>& dx, const Tensor<Scalar>& dy, const Tensor<Scalar>& x,
                         const Tensor<Scalar>& y, bool accumulate) const {
+    if (dy.dev()->kind() == CPU) {
+      host::nonlin_backward<Scalar>(code(), static_cast<int>(dy.rows()), static_cast<int>(dy.cols()), dy.data(),
+                                   x.size() > 0 ? x.data() : nullptr, y.size() > 0 ? y.data() : nullptr, dx.data(),
+                                   accumulate);
+      return;
+    }
     internal::require_gpu(dy.dev(), "NonlinOp::backward");
     GINN_HIP_CALL(ginn_hip_nonlin_bwd(internal::ctx_of(dy), dtype_of<Scalar>(), code(),
                                       static_cast<int>(dy.rows()), static_cast<int>(dy.cols()), dy.data(),

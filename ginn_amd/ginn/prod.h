@@ -6,6 +6,7 @@
 #ifndef GINN_PROD_H
 #define GINN_PROD_H
 
+#include <ginn/cpu_ops.h>
 #include <ginn/tensor.h>
 
 namespace ginn {
@@ -99,6 +100,49 @@ inline void gpu_batched_prod(Tensor<Scalar>& c, Tensor<Scalar>& a, Tensor<Scalar
                            static_cast<int>(a_inner), static_cast<int>(b_outer), static_cast<int>(batches),
                            res == ProdResult::Add ? Scalar(1.f) : Scalar(0.f), ta ? OP_T : OP_N,
                            tb ? OP_T : OP_N);
+}
+
+// The same two products for tensors on cpu(): the host layer's own loops (ginn/cpu_ops.h), where the
+// reference contracts with Eigen (ginn/node/prod.h:31-34,46-51).
+template <typename Scalar>
+inline void cpu_prod(Tensor<Scalar>& c, Tensor<Scalar>& a, Tensor<Scalar>& b, ProdResult res = ProdResult::Assign,
+                     ProdTranspose tra = ProdTranspose::None) {
+  const bool ta = tra == ProdTranspose::First || tra == ProdTranspose::Both;
+  const bool tb = tra == ProdTranspose::Second || tra == ProdTranspose::Both;
+  const Size a_outer = ta ? a.cols() : a.rows(), a_inner = ta ? a.rows() : a.cols();
+  const Size b_outer = tb ? b.rows() : b.cols(), b_inner = tb ? b.cols() : b.rows();
+  GINN_ASSERT(a_inner == b_inner);
+  GINN_ASSERT(a_outer == c.rows());
+  GINN_ASSERT(b_outer == c.cols());
+  if constexpr (is_floating_point_v<Scalar>) {
+    host::gemm<Scalar>(ta, tb, static_cast<int>(a_outer), static_cast<int>(b_outer), static_cast<int>(a_inner), a.data(),
+                      static_cast<int>(a.rows()), b.data(), static_cast<int>(b.rows()),
+                      res == ProdResult::Add ? 1.f : 0.f, c.data(), static_cast<int>(c.rows()));
+  } else {
+    GINN_THROW("Unexpected Scalar type in cpu_prod!");
+  }
+}
+template <typename Scalar>
+inline void cpu_batched_prod(Tensor<Scalar>& c, Tensor<Scalar>& a, Tensor<Scalar>& b,
+                             ProdResult res = ProdResult::Assign, ProdTranspose tra = ProdTranspose::None) {
+  const Shape as = Tensor<Scalar>::reduce(a.shape(), 3), bs = Tensor<Scalar>::reduce(b.shape(), 3),
+              cs = Tensor<Scalar>::reduce(c.shape(), 3);
+  const bool ta = tra == ProdTranspose::First || tra == ProdTranspose::Both;
+  const bool tb = tra == ProdTranspose::Second || tra == ProdTranspose::Both;
+  const Size a_outer = ta ? as[1] : as[0], a_inner = ta ? as[0] : as[1];
+  const Size b_outer = tb ? bs[0] : bs[1], b_inner = tb ? bs[1] : bs[0];
+  GINN_ASSERT(a_inner == b_inner);
+  GINN_ASSERT(a_outer == cs[0]);
+  GINN_ASSERT(b_outer == cs[1]);
+  if constexpr (is_floating_point_v<Scalar>) {
+    for (Size i = 0; i < as[2]; ++i)
+      host::gemm<Scalar>(ta, tb, static_cast<int>(a_outer), static_cast<int>(b_outer), static_cast<int>(a_inner),
+                        a.data() + i * as[0] * as[1], static_cast<int>(as[0]), b.data() + i * bs[0] * bs[1],
+                        static_cast<int>(bs[0]), res == ProdResult::Add ? 1.f : 0.f, c.data() + i * cs[0] * cs[1],
+                        static_cast<int>(cs[0]));
+  } else {
+    GINN_THROW("Unexpected Scalar type in cpu_batched_prod!");
+  }
 }
 
 }  // namespace internal

@@ -18,13 +18,16 @@ using namespace ginn;
 namespace {
 
 thread_local std::string g_error;
+// Where the node cases below place their data: the HIP device, or cpu() for the host layer's own loops
+// (shim_use_device).
+bool g_on_cpu = false;
 
 template <typename S>
 Ptr<DataNode<S>> make_data(const Shape& shape, const float* vals, bool has_grad) {
   auto x = Data<S>(cpu(), shape);
   S* p = x->value().v();
   for (Size i = 0; i < x->value().size(); ++i) p[i] = S(vals[i]);
-  x->move_to(gpu());
+  if (!g_on_cpu) x->move_to(gpu());
   x->set_has_grad(has_grad);
   return x;
 }
@@ -51,7 +54,7 @@ void run_masked(const NodePtr<S>& e1, const NodePtr<S>& e2, const float* mask, f
   g.forward();
   g.reset_grad();
   g.backward(1.);
-  gpu()->synchronize();
+  if (!g_on_cpu) gpu()->synchronize();
 }
 
 template <typename S>
@@ -150,6 +153,10 @@ extern "C" {
 const char* shim_last_error() { return g_error.c_str(); }
 
 int shim_gpus() { return gpus(); }
+
+// 1: shim_prod_node, shim_affine_node, shim_nonlin_node and shim_mlp_on_cpu keep their graphs on cpu();
+// 0 (the default): on the HIP device.
+void shim_use_device(int on_cpu) { g_on_cpu = on_cpu != 0; }
 
 int shim_prod_node(int dtype, int batched, const long* a_dims, int a_rank, const long* b_dims, int b_rank,
                    const float* a, const float* b, const float* mask, float* out_value, float* out_da,

@@ -54,10 +54,19 @@ def test_data_and_weight_nodes(ginn):
     assert not w.has_grad
 
 
-def test_compute_without_a_device_fails_loudly(ginn):
+def test_nodes_on_cpu_compute_or_fail_loudly(ginn):
+    """The product-path nodes have host forms on cpu() (the same graph code as on the device); every other
+    node refuses a cpu() tensor instead of computing something else."""
     x = ginn.Data(np.ones((2, 2)))
+    s = ginn.Sigmoid(x)
+    s.forward()
+    assert s.value.list() == pytest.approx([1 / (1 + np.exp(-1.0))] * 4, rel=1e-6)
+    W = ginn.Data(np.array([[1.0, 2.0], [3.0, 4.0]]))
+    p = ginn.Prod(W, x)
+    p.forward()
+    assert p.value.list() == [3.0, 7.0, 3.0, 7.0]
     with pytest.raises(RuntimeError, match="HIP device only"):
-        ginn.Sigmoid(x).forward()
+        ginn.LayerNorm(x).forward()
 
 
 @pytest.mark.gpu
