@@ -90,7 +90,9 @@ struct StripParams {
   int strips;
 };
 
-// NB: direct loads of B per buffer (each brings 256 bytes of K for four columns): 1, 2, 4 for n <= 4, 8, 16.
+// NB: direct loads of B per buffer (each brings 256 bytes of K for four columns): ceil(n / 4), so that every
+// load instruction has at least one active lane -- one whose lanes are all beyond n would be branched around,
+// and the waits below count load instructions.
 template <typename T, int NB, bool GENERAL>
 __global__ __launch_bounds__(kThreads) void gemm_strip_kernel(StripParams p) {
   using S = typename T::storage;
@@ -318,6 +320,7 @@ template <typename T>
 int launch_width(ginn_hip_ctx* ctx, const StripParams& p, bool general) {
   if (p.n <= 4) return launch_general<T, 1>(ctx, p, general);
   if (p.n <= 8) return launch_general<T, 2>(ctx, p, general);
+  if (p.n <= 12) return launch_general<T, 3>(ctx, p, general);
   return launch_general<T, 4>(ctx, p, general);
 }
 

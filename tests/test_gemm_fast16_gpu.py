@@ -484,7 +484,7 @@ def test_masked_tile_edges_of_the_small_slice_kernel(dev, dt, op_a, op_b, m, n, 
 
 
 @pytest.mark.parametrize("dt", [capi.F16, capi.BF16, capi.F32])
-@pytest.mark.parametrize("n", [1, 2, 3, 5, 8, 9, 16])
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 8, 9, 12, 13, 16])
 @pytest.mark.parametrize("m,k", [(2048, 1024), (4096, 4096), (2056, 1040), (4104, 2064), (2048, 8208), (4096, 1040),
                                  (4104, 1056)])
 @pytest.mark.parametrize("beta", [0.0, 0.5])
