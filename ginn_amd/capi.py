@@ -59,6 +59,10 @@ PROTOTYPES = {
     "ginn_hip_gemm_strided_batched": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                               c_void_p, c_int, c_longlong, c_void_p, c_int, c_longlong,
                                               c_float, c_void_p, c_int, c_longlong, c_int]),
+    "ginn_hip_gemm_strided_batched2": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                               c_void_p, c_int, c_longlong, c_longlong, c_void_p, c_int, c_longlong,
+                                               c_longlong, c_float, c_void_p, c_int, c_longlong, c_longlong, c_int,
+                                               c_int]),
     "ginn_hip_gemm_grouped": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int,
                                       POINTER(c_void_p), POINTER(c_int), POINTER(c_int), c_float,
                                       POINTER(c_void_p), POINTER(c_int)]),

@@ -388,6 +388,11 @@ struct GemmArgs {
   int ldc;
   long long stride_c;
   int batch;
+  // Two-level batch (batch_inner > 0): slice z of the `batch` slices lies at
+  // (z % batch_inner) * stride + (z / batch_inner) * stride2 of each operand.  Only launch_gemm_bsmall
+  // reads these; ginn_hip_gemm_strided_batched2 runs everything else level by level.
+  int batch_inner = 0;
+  long long stride_a2 = 0, stride_b2 = 0, stride_c2 = 0;
   // Optional epilogue: C = act(acc + beta*C + bias[row]); `pre` (same ld and
   // stride as C) receives the value before the activation.
   const void* bias = nullptr;

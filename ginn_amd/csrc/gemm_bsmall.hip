@@ -31,6 +31,9 @@ struct Params {
   int m, n, k;
   int lda, ldb, ldc;
   long long sa, sb, sc;
+  // slice z at (z % inner) * s + (z / inner) * s2 (inner = batch for a plain strided batch)
+  long long sa2, sb2, sc2;
+  int inner;
   int tiles_m, tiles_n;  // per slice
   int batch;
   int whole_lines;  // columns of C start on 128-byte lines
@@ -68,8 +71,9 @@ __global__ __launch_bounds__(kThreadsB) void gemm_bsmall_kernel(Params p) {
     const int per = (tiles * p.batch) >> 3;
     pid = (pid & 7) * per + (pid >> 3);
   }
-  const long long bz = pid / tiles;
+  const int bz = pid / tiles;
   const int tile = pid % tiles;
+  const long long z_in = bz % p.inner, z_out = bz / p.inner;
   const int m0 = (tile % p.tiles_m) * G::BM, n0 = (tile / p.tiles_m) * G::BN;
   const int KT = (p.k + BK - 1) / BK;
   // K values in the last K tile (64 unless K is no multiple of the tile): the lanes whose 16 bytes of that
@@ -103,9 +107,11 @@ __global__ __launch_bounds__(kThreadsB) void gemm_bsmall_kernel(Params p) {
   const long long a_kstep = (AKC ? (long long)BK : (long long)BK * p.lda) * ES;
   const long long b_kstep = (BKC ? (long long)BK : (long long)BK * p.ldb) * ES;
   const char* a_next =
-      static_cast<const char*>(p.A) + (bz * p.sa + (AKC ? (long long)m0 * p.lda : (long long)m0)) * ES;
+      static_cast<const char*>(p.A) +
+      (z_in * p.sa + z_out * p.sa2 + (AKC ? (long long)m0 * p.lda : (long long)m0)) * ES;
   const char* b_next =
-      static_cast<const char*>(p.B) + (bz * p.sb + (BKC ? (long long)n0 * p.ldb : (long long)n0)) * ES;
+      static_cast<const char*>(p.B) +
+      (z_in * p.sb + z_out * p.sb2 + (BKC ? (long long)n0 * p.ldb : (long long)n0)) * ES;
   auto issue_tile = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < kPassA; ++i) {
@@ -255,7 +261,7 @@ __global__ __launch_bounds__(kThreadsB) void gemm_bsmall_kernel(Params p) {
 
   // ---- epilogue: round, stage through the wave's own LDS slice (the last
   // barrier above freed the stages), store 16-byte column segments.
-  uint16_t* C = static_cast<uint16_t*>(p.C) + bz * p.sc;
+  uint16_t* C = static_cast<uint16_t*>(p.C) + z_in * p.sc + z_out * p.sc2;
   char* stage = lds + wave * G::kEpiWaveBytes;
   const int l32 = lane & 31, lhi = lane >> 5;
 #pragma unroll
@@ -344,6 +350,8 @@ int launch_gemm_bsmall(ginn_hip_ctx* ctx, const GemmArgs& a) {
   const bool slim = a.k == 64 || a.m == 64 || a.n == 64;
   if (!slim || a.m > 1024 || a.n > 1024 || a.k > 1024) return kUnsupported;
   if (a.lda % 8 || a.ldb % 8 || a.ldc % 8 || a.stride_a % 8 || a.stride_b % 8 || a.stride_c % 8) return kUnsupported;
+  const bool two_level = a.batch_inner > 0;
+  if (two_level && (a.stride_a2 % 8 || a.stride_b2 % 8 || a.stride_c2 % 8 || a.batch % a.batch_inner)) return kUnsupported;
   auto aligned16 = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
   if (!aligned16(a.A) || !aligned16(a.B) || !aligned16(a.C)) return kUnsupported;
   if ((long long)a.lda * 128 * 2 >= (1ll << 31) || (long long)a.ldb * 128 * 2 >= (1ll << 31)) return kUnsupported;
@@ -364,10 +372,14 @@ int launch_gemm_bsmall(ginn_hip_ctx* ctx, const GemmArgs& a) {
   p.sa = a.stride_a;
   p.sb = a.stride_b;
   p.sc = a.stride_c;
+  p.inner = two_level ? a.batch_inner : a.batch;
+  p.sa2 = two_level ? a.stride_a2 : 0;
+  p.sb2 = two_level ? a.stride_b2 : 0;
+  p.sc2 = two_level ? a.stride_c2 : 0;
   p.tiles_m = (a.m + 64 * fm - 1) / (64 * fm);
   p.tiles_n = (a.n + 64 * fn - 1) / (64 * fn);
   p.batch = a.batch;
-  p.whole_lines = a.ldc % 64 == 0 && a.stride_c % 64 == 0 && reinterpret_cast<uintptr_t>(a.C) % 128 == 0;
+  p.whole_lines = a.ldc % 64 == 0 && a.stride_c % 64 == 0 && p.sc2 % 64 == 0 && reinterpret_cast<uintptr_t>(a.C) % 128 == 0;
   const long long blocks = (long long)p.tiles_m * p.tiles_n * a.batch;
   if (blocks < ctx->num_cus || blocks > (1ll << 30)) return kUnsupported;
   p.xcd_spread = blocks % 8 == 0 ? 1 : 0;

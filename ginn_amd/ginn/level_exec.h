@@ -25,6 +25,7 @@
 #include <cstring>
 #include <functional>
 #include <utility>
+#include <unordered_set>
 
 #include <ginn/node.h>
 
@@ -127,6 +128,9 @@ class LevelExecutor {
   // that fill is in no plan, so the passes cannot be replayed from plans.
   bool unplanned_fill_ = false;
   bool frozen_ = false;
+  // Nodes that postpone the kernel behind their value (PostponedValue) and have a reader whose work a
+  // frozen pass replays from the recording: asked for their value right after forward() (freeze()).
+  std::unordered_set<BaseNode*> settle_after_forward_;
   ginn_hip_graph* pass_graph_ = nullptr;  // a recorded frozen pass (record_pass())
 
   void drop_graph() {
@@ -679,6 +683,7 @@ class LevelExecutor {
         if (pass == kForward) {
           n->forwarded = false;
           n->forward();
+          settle_if_replayed_reader(n);
         } else if (pass == kReset) {
           n->reset_grad();
         } else {
@@ -688,6 +693,24 @@ class LevelExecutor {
       if (it.plan >= 0) launch(plans_[pass][static_cast<size_t>(it.plan)], it.first, it.count);
       if (it.chain >= 0) launch_chain(chains_[static_cast<size_t>(it.chain)]);
     }
+  }
+
+  // freeze(): which nodes with a postponed value are read by a node that does not run itself in the frozen
+  // forward pass (its work is replayed from the recording, so it never calls value()).
+  void find_replayed_readers() {
+    settle_after_forward_.clear();
+    std::unordered_set<const BaseNode*> runs_itself;
+    for (const Step& step : steps_[kForward])
+      for (BaseNode* n : step.direct) runs_itself.insert(n);
+    for (auto& n : list_) {
+      if (runs_itself.count(n.get())) continue;
+      for (auto& in : n->ins())
+        if (dynamic_cast<PostponedValue*>(in.get())) settle_after_forward_.insert(in.get());
+    }
+  }
+  void settle_if_replayed_reader(BaseNode* n) {
+    if (!settle_after_forward_.empty() && settle_after_forward_.count(n))
+      dynamic_cast<PostponedValue*>(n)->settle_value();
   }
 
   void seed_sink(double loss_coeff) {
@@ -746,6 +769,7 @@ class LevelExecutor {
                 "LevelExecutor::freeze(): a node that declares GradUse::Overwrites added to a gradient that "
                 "reset_grad() had only flagged; run with set_lazy_grad_reset(false)");
     plan_late_reductions();
+    find_replayed_readers();
     frozen_ = true;
     return *this;
   }
@@ -832,6 +856,7 @@ class LevelExecutor {
         for (BaseNode* n : step.direct) {
           n->forwarded = false;
           n->forward();
+          settle_if_replayed_reader(n);
         }
         if (step.plan >= 0) launch(plans_[kForward][static_cast<size_t>(step.plan)]);
       }

@@ -260,7 +260,8 @@ class Node : public BaseNode {
 
   void init_grad() override {
     GINN_ASSERT(forwarded, "Cannot init grad on non-forwarded nodes!");
-    if (has_grad() && value().size() != grad().size()) grad().resize(value().shape());
+    // shape(), not value(): a node that postpones the kernel behind its value is not asked for it here
+    if (has_grad() && this->size() != grad().size()) grad().resize(this->shape());
   }
   void reset_grad() override {
     init_grad();
@@ -550,6 +551,17 @@ class PendingInPlace {
   // so that the storage written over holds the final contents for any reader
   // once forward() has returned (ginn/node/inplace.h:104-123, 152-212).
   virtual void settle() = 0;
+};
+
+// A node that postpones the kernel behind its value until value() is called (LayerNorm, Permute,
+// BatchedProd), so that the node reading it can do both steps in one.  Every reader that runs as code of
+// its own calls value() and gets it.  A frozen LevelExecutor replays the work of all other readers from
+// what it recorded, calling nothing: it therefore asks such a node for its value right after forward()
+// when one of the node's readers is among the replayed ones (settle_value()).
+class PostponedValue {
+ public:
+  virtual ~PostponedValue() = default;
+  virtual void settle_value() = 0;
 };
 
 class Graph {

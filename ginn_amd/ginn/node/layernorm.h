@@ -19,7 +19,7 @@ class CwiseProdAddNode;
 // gradient has no other user, both backward steps as one
 // (ginn_hip_layernorm_affine_bwd).  Any other reader gets the value as usual.
 template <typename Scalar>
-class LayerNormNode : public BaseDataNode<Scalar> {
+class LayerNormNode : public BaseDataNode<Scalar>, public PostponedValue {
   friend class CwiseProdAddNode<Scalar>;
 
  protected:
@@ -75,6 +75,7 @@ class LayerNormNode : public BaseDataNode<Scalar> {
   }
   using Node<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
+  void settle_value() override { (void)std::as_const(*this).value(); }
   Shape shape() const override { return pending_ ? in_->shape() : value().shape(); }
   DevPtr dev() const override { return in_->dev(); }
   BaseNode::GradUse grad_use(size_t) const override { return BaseNode::GradUse::Overwrites; }

@@ -5,6 +5,7 @@
 #define GINN_NODE_LAYOUT_H
 
 #include <ginn/node/data.h>
+#include <ginn/node/slices.h>
 #include <ginn/nonlin.h>
 
 namespace ginn {
@@ -514,12 +515,19 @@ GINN_MAKE_SCALAR_FORWARDING_FACTORY(Map);
 
 // Axis permutation: result extent k is the input's extent indices[k]
 // (ginn/node/layout.h:723-821); backward adds the inversely permuted gradient.
+// On the HIP device the copy is postponed until the value is read when the
+// result's slices are matrices inside the input's memory (node/slices.h): a
+// BatchedProd that multiplies them takes them from there (and puts the gradient
+// there), and a BatchedProd in front whose product is still pending writes its
+// result permuted; every other reader gets the copy as usual.
 template <typename Scalar>
-class PermuteNode : public BaseDataNode<Scalar> {
+class PermuteNode : public BaseDataNode<Scalar>, public internal::SliceProvider<Scalar>, public PostponedValue {
  protected:
   NodePtr<Scalar> in_;
   Shape indices_;
   bool overwrite_ = false;  // set by InPlacePermuteNode: results replace, through a temporary
+  mutable bool pending_ = false;  // forward() has run, the copy has not
+  bool skip_backward_ = false;    // the only user has put the gradient into the input's already
 
   static Shape permute(const Shape& s, const Shape& perm) {
     Shape out(s.size());
@@ -547,13 +555,50 @@ class PermuteNode : public BaseDataNode<Scalar> {
     GINN_HIP_CALL(ginn_hip_permute(internal::ctx_of(dst), dtype_of<Scalar>(), static_cast<int>(dims.size()),
                                    dims.data(), p.data(), src.data(), dst.data(), accumulate ? 1 : 0));
   }
+  Tensor<Scalar>& raw_value() const { return const_cast<Tensor<Scalar>&>(BaseDataNode<Scalar>::value()); }
+  internal::SliceTaker<Scalar>* pending_product() const {
+    auto* t = dynamic_cast<internal::SliceTaker<Scalar>*>(in_.get());
+    return t && t->product_pending() ? t : nullptr;
+  }
+  // The result's slices as matrices inside `stored`, which holds the input (forward: its value) or has the
+  // input's shape (backward: its gradient).
+  bool slices_in_input(Scalar* stored, internal::BatchView<Scalar>& v) const {
+    return internal::permuted_slices(stored, in_->shape(), indices_, v);
+  }
+  // The input's slices as matrices inside `stored`, which has the result's shape.
+  bool slices_in_result(Tensor<Scalar>& stored, internal::BatchView<Scalar>& v) const {
+    return internal::permuted_slices(stored.data(), stored.shape(), inverse(indices_), v);
+  }
+  void copy_now() const {
+    if (auto* t = pending_product()) {  // the product in front writes its slices where the copy would put them
+      internal::BatchView<Scalar> v;
+      if (slices_in_result(raw_value(), v)) {
+        t->produce_into(v);
+        return;
+      }
+    }
+    run(in_->value(), in_->shape(), indices_, raw_value(), false);
+  }
   void forward_() override {
-    const Shape s = in_->value().shape();
+    const Shape s = in_->shape();
     check_permutation(s);
-    value().resize(permute(s, indices_));
-    run(in_->value(), s, indices_, value(), false);
+    raw_value().resize(permute(s, indices_));
+    internal::BatchView<Scalar> v;
+    const bool on_gpu = this->dev()->kind() == GPU;
+    if (on_gpu && !overwrite_ && is_floating_point_v<Scalar> && raw_value().size() > 0 &&
+        (internal::permuted_slices(static_cast<Scalar*>(nullptr), s, indices_, v) ||
+         (pending_product() && slices_in_result(raw_value(), v)))) {
+      pending_ = true;
+      return;
+    }
+    pending_ = false;
+    copy_now();
   }
   void backward_() override {
+    if (skip_backward_) {
+      skip_backward_ = false;
+      return;
+    }
     if (!in_->has_grad()) return;
     if (overwrite_) {
       // grad() is in's gradient storage under the permuted shape: permute into a
@@ -565,15 +610,45 @@ class PermuteNode : public BaseDataNode<Scalar> {
       flat = tmp;
     } else {
       const bool fresh = in_->take_lazy_zero();
+      // The only user of a batched product's gradient: the product reads it from here, permuted.
+      if (fresh)
+        if (auto* t = dynamic_cast<internal::SliceTaker<Scalar>*>(in_.get())) {
+          internal::BatchView<Scalar> v;
+          if (slices_in_result(grad(), v) && t->take_grad_slices(v)) return;
+        }
       run(grad(), grad().shape(), inverse(indices_), in_->grad(), !fresh);
     }
   }
 
  public:
-  using BaseDataNode<Scalar>::value;
+  const Tensor<Scalar>& value() const override {
+    if (pending_) {
+      pending_ = false;
+      copy_now();
+    }
+    return BaseDataNode<Scalar>::value();
+  }
+  using Node<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
+  void settle_value() override { (void)std::as_const(*this).value(); }
+  Shape shape() const override { return BaseDataNode<Scalar>::value().shape(); }
+  DevPtr dev() const override { return BaseDataNode<Scalar>::value().dev(); }
   BaseNode::GradUse grad_use(size_t) const override {
     return overwrite_ ? BaseNode::GradUse::Accumulates : BaseNode::GradUse::Overwrites;
+  }
+  bool value_slices(internal::BatchView<Scalar>& v) override {
+    if (!pending_ || pending_product()) return false;
+    return slices_in_input(in_->value().data(), v);
+  }
+  bool grad_slices(internal::BatchView<Scalar>& v, bool& accumulate) override {
+    if (overwrite_ || !in_->has_grad() || this->dev()->kind() != GPU) return false;
+    internal::BatchView<Scalar> probe;
+    if (!internal::permuted_slices(static_cast<Scalar*>(nullptr), in_->shape(), indices_, probe)) return false;
+    const bool fresh = in_->take_lazy_zero();  // before grad(): a flagged gradient would be cleared on sight
+    slices_in_input(in_->grad().data(), v);
+    accumulate = !fresh;
+    skip_backward_ = true;
+    return true;
   }
   PermuteNode(const NodePtr<Scalar>& in, Shape indices)
       : BaseDataNode<Scalar>({in}), in_(in), indices_(std::move(indices)) {}

@@ -6,6 +6,7 @@
 #include <atomic>
 
 #include <ginn/node/data.h>
+#include <ginn/node/slices.h>
 #include <ginn/nonlin.h>
 #include <ginn/prod.h>
 
@@ -328,9 +329,26 @@ class GatherProdNode : public BaseDataNode<Scalar>, public ColumnPartition {
 GINN_MAKE_SCALAR_FORWARDING_FACTORY(GatherProd);
 
 // Per-slice product over all trailing dimensions (rank >= 3 inputs).
+// On the HIP device the product is carried out when its value is first read: an operand that is a Permute
+// whose copy is still pending is then read through its slices in ITS input's memory, and a Permute right
+// behind this node has the result written permuted (node/slices.h); the gradients take the same ways back.
 template <typename Scalar>
-class BatchedProdNode : public BaseDataNode<Scalar> {
+class BatchedProdNode : public BaseDataNode<Scalar>, public internal::SliceTaker<Scalar>, public PostponedValue {
   NodePtr<Scalar> a_, b_;
+  mutable bool pending_ = false;  // forward() has run, the product has not
+  bool grad_elsewhere_ = false;   // this pass's gradient lies in grad_view_ (take_grad_slices)
+  internal::BatchView<Scalar> grad_view_;
+
+  Tensor<Scalar>& raw_value() const { return const_cast<Tensor<Scalar>&>(BaseDataNode<Scalar>::value()); }
+  // The slices of an operand's value: those a pending Permute offers, or the operand's own tensor.
+  static internal::BatchView<Scalar> operand(const NodePtr<Scalar>& x) {
+    internal::BatchView<Scalar> v;
+    if (auto* p = dynamic_cast<internal::SliceProvider<Scalar>*>(x.get()); p && p->value_slices(v)) return v;
+    return internal::contiguous_slices(x->value());
+  }
+  void multiply_into(const internal::BatchView<Scalar>& out) const {
+    internal::batched_product(internal::ctx_of(raw_value()), out, operand(a_), false, operand(b_), false, false);
+  }
 
   void forward_() override {
     const Shape sa = a_->shape(), sb = b_->shape();
@@ -341,13 +359,15 @@ class BatchedProdNode : public BaseDataNode<Scalar> {
       GINN_ASSERT(sa[i] == sb[i], "Mismatching batch dimensions in BatchedProd!");
     Shape s = sb;
     s[0] = sa[0];
-    value().resize(s);
+    raw_value().resize(s);
+    grad_elsewhere_ = false;
     if (dev()->kind() == CPU) {
-      internal::cpu_batched_prod(value(), a_->value(), b_->value());
+      pending_ = false;
+      internal::cpu_batched_prod(raw_value(), a_->value(), b_->value());
       return;
     }
     internal::require_gpu(dev(), "BatchedProd");
-    internal::gpu_batched_prod(value(), a_->value(), b_->value());
+    pending_ = raw_value().size() > 0;
   }
   void backward_() override {
     using namespace internal;
@@ -360,22 +380,57 @@ class BatchedProdNode : public BaseDataNode<Scalar> {
                          b_->take_lazy_zero() ? ProdResult::Assign : ProdResult::Add, ProdTranspose::First);
       return;
     }
-    if (a_->has_grad()) {
-      const bool fresh = a_->take_lazy_zero();
-      gpu_batched_prod(a_->grad(), grad(), b_->value(), fresh ? ProdResult::Assign : ProdResult::Add,
-                       ProdTranspose::Second);
+    const BatchView<Scalar> dy = grad_elsewhere_ ? grad_view_ : contiguous_slices(grad());
+    grad_elsewhere_ = false;
+    ginn_hip_ctx* ctx = ctx_of(raw_value());
+    // Where the gradient of an operand goes: into the slices a Permute names inside its input's gradient
+    // (this node being the only user of the Permute's), or into the operand's own gradient tensor.
+    auto target = [](const NodePtr<Scalar>& x, bool& accumulate) {
+      const bool fresh = x->take_lazy_zero();
+      BatchView<Scalar> v;
+      if (fresh)
+        if (auto* p = dynamic_cast<SliceProvider<Scalar>*>(x.get()); p && p->grad_slices(v, accumulate)) return v;
+      accumulate = !fresh;
+      return contiguous_slices(x->grad());
+    };
+    if (a_->has_grad()) {  // dA = dY B^T
+      bool acc = false;
+      const BatchView<Scalar> da = target(a_, acc);
+      batched_product(ctx, da, dy, false, operand(b_), true, acc);
     }
-    if (b_->has_grad()) {
-      const bool fresh = b_->take_lazy_zero();
-      gpu_batched_prod(b_->grad(), a_->value(), grad(), fresh ? ProdResult::Assign : ProdResult::Add,
-                       ProdTranspose::First);
+    if (b_->has_grad()) {  // dB = A^T dY
+      bool acc = false;
+      const BatchView<Scalar> db = target(b_, acc);
+      batched_product(ctx, db, operand(a_), true, dy, false, acc);
     }
   }
 
  public:
-  using BaseDataNode<Scalar>::dev;
-  using BaseDataNode<Scalar>::value;
   using BaseDataNode<Scalar>::grad;
+  const Tensor<Scalar>& value() const override {
+    if (pending_) {
+      pending_ = false;
+      multiply_into(internal::contiguous_slices(raw_value()));
+    }
+    return BaseDataNode<Scalar>::value();
+  }
+  using Node<Scalar>::value;
+  void settle_value() override { (void)std::as_const(*this).value(); }
+  Shape shape() const override { return BaseDataNode<Scalar>::value().shape(); }
+  DevPtr dev() const override { return BaseDataNode<Scalar>::value().dev(); }
+
+  bool product_pending() const override { return pending_; }
+  void produce_into(const internal::BatchView<Scalar>& v) override {
+    GINN_ASSERT(pending_, "BatchedProd: no product is pending");
+    pending_ = false;
+    multiply_into(v);
+  }
+  bool take_grad_slices(const internal::BatchView<Scalar>& v) override {
+    if (dev()->kind() != GPU) return false;
+    grad_view_ = v;
+    grad_elsewhere_ = true;
+    return true;
+  }
 
   BatchedProdNode(const NodePtr<Scalar>& a, const NodePtr<Scalar>& b)
       : BaseDataNode<Scalar>({a, b}), a_(a), b_(b) {}

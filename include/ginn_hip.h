@@ -219,6 +219,26 @@ int ginn_hip_gemm_strided_batched(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
                                   long long stride_b, float beta, void* C,
                                   int ldc, long long stride_c, int batch);
 
+/* The same with the slices numbered in two levels: slice z, z < batch_inner *
+ * batch_outer, of an operand lies at base + (z % batch_inner) * stride +
+ * (z / batch_inner) * stride2.  This is how the [rows x cols] slices of a
+ * rank-4 tensor lie in memory AFTER a permutation of its axes that keeps (or
+ * swaps) the first two: BatchedProdNode (ginn/node/prod.h:104-187) reads the
+ * heads of an attention layer where the projection wrote them, and writes its
+ * result where the next projection reads it, instead of through PermuteNode
+ * copies (ginn/node/layout.h:723-821; examples/min-gpt.cu.cpp:117-135).  One
+ * launch where the small-slice kernel takes the shape, batch_outer strided
+ * batches otherwise. */
+int ginn_hip_gemm_strided_batched2(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
+                                   ginn_hip_op op_a, ginn_hip_op op_b, int m,
+                                   int n, int k, const void* A, int lda,
+                                   long long stride_a, long long stride_a2,
+                                   const void* B, int ldb, long long stride_b,
+                                   long long stride_b2, float beta, void* C,
+                                   int ldc, long long stride_c,
+                                   long long stride_c2, int batch_inner,
+                                   int batch_outer);
+
 /* ginn_hip_gemm for callers that cannot allocate: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference (whose BLAS handle allocates its workspace

@@ -122,6 +122,77 @@ int lazy_graph(int mode, int passes, int hs, int nh, int B, int T, int V, const 
   return 0;
 }
 
+// Batched products on permuted views (node/slices.h): X [C x B T] is projected three times (Prod with Wk, Wq,
+// Wv [C x C], C = hs nh), each projection reshaped to [hs, nh, B, T] and permuted to the slices of a head
+// (k: [T, hs, B, nh], q and v: [hs, T, B, nh]); s = BatchedProd(k, q), y = BatchedProd(v, s), y permuted back to
+// [hs, nh, B, T] and reshaped to [C x B T]; loss = Sum(mask (*) y).  Pass 1 runs on x1, then x2 is written into
+// the SAME input tensor and pass 2 runs (a frozen executor replays; a value that was postponed and never asked
+// for would show up as pass 1's).  mode: 0 = Graph, 1 = executor, 2 = frozen executor, 3 = frozen and recorded
+// as a device graph.  read: 1 = the values of k and of s are read back between forward and backward of pass 2
+// (the postponed copy / product must then run, and everything still agree).  Outputs of pass 2: y, dX, dWk,
+// dWq, dWv; *out_kernels: kernel launches of the recorded pass (mode 3).
+template <typename S>
+int permuted_products(int mode, int read, int hs, int nh, int B, int T, const float* x1, const float* x2,
+                      const float* const* w, const float* mask, float* out_y, float* out_dx, float* const* out_dw,
+                      float* out_k, float* out_s, long* out_kernels) {
+  const Size C = static_cast<Size>(hs) * nh, N = static_cast<Size>(B) * T;
+  auto X = data_of<S>({C, N}, x1, true);
+  std::vector<Ptr<WeightNode<S>>> W;
+  for (int i = 0; i < 3; ++i) W.push_back(weight_of<S>({C, C}, w[i]));
+  auto M = data_of<S>({C, N}, mask, false);
+  auto heads = [&](int i, Shape perm) -> NodePtr<S> {
+    NodePtr<S> proj = Prod(NodePtr<S>(W[i]), NodePtr<S>(X));
+    return Permute(NodePtr<S>(Reshape(proj, Shape{hs, nh, B, T})), std::move(perm));
+  };
+  NodePtr<S> k = heads(0, {3, 0, 2, 1}), q = heads(1, {0, 3, 2, 1}), v = heads(2, {0, 3, 2, 1});
+  NodePtr<S> s = BatchedProd(k, q);
+  NodePtr<S> y = Permute(NodePtr<S>(BatchedProd(v, s)), Shape{0, 3, 2, 1});
+  NodePtr<S> flat = Reshape(y, Shape{C, N});
+  auto loss = Sum(CwiseProd(flat, NodePtr<S>(M)));
+  Graph g(loss);
+  auto set_input = [&](const float* vals) {
+    Tensor<S> host(cpu(), X->value().shape());
+    for (Size i = 0; i < host.size(); ++i) host.v()[i] = S(vals[i]);
+    X->value() = host.copy_to(gpu());  // same size: copies into the tensor's storage
+  };
+  auto pass = [&](auto& runner, bool look) {
+    runner.reset_forwarded();
+    runner.forward();
+    if (look) {
+      read_back(k->value(), out_k);
+      read_back(s->value(), out_s);
+    }
+    runner.reset_grad();
+    runner.backward(1.);
+  };
+  if (mode == 0) {
+    pass(g, false);
+    set_input(x2);
+    pass(g, read != 0);
+  } else {
+    LevelExecutor ex(g);
+    pass(ex, false);
+    if (mode >= 2) ex.freeze();
+    set_input(x2);
+    if (mode == 3) {
+      ex.record_pass();
+      if (out_kernels) *out_kernels = static_cast<long>(ex.recorded_kernels());
+      ex.replay_pass();
+      if (read) {
+        read_back(k->value(), out_k);
+        read_back(s->value(), out_s);
+      }
+    } else {
+      pass(ex, read != 0);
+    }
+  }
+  gpu()->synchronize();
+  read_back(flat->value(), out_y);
+  read_back(X->grad(), out_dx);
+  for (int i = 0; i < 3; ++i) read_back(W[i]->grad(), out_dw[i]);
+  return 0;
+}
+
 }  // namespace
 
 #define DISPATCH(DTYPE, CALL)                                     \
@@ -163,6 +234,29 @@ void shim_set_beside_pass(int on) { set_beside_pass(on != 0); }
 // the pass's stream) and an operand of an Add; V [d x d] has the large product as its only user.
 // Three passes; out_dw / out_dv: the gradients of W and V after the last one.  out_beside: launches
 // that went to the second stream.  mode: 0 = Graph, 1 = executor, 2 = frozen executor.
+int shim_permuted_products(int dtype, int mode, int read, int hs, int nh, int B, int T, const float* x1, const float* x2,
+                           const float* const* w, const float* mask, float* out_y, float* out_dx,
+                           float* const* out_dw, float* out_k, float* out_s, long* out_kernels) {
+  try {
+    switch (dtype) {
+      case GINN_HIP_F32:
+        return permuted_products<Real>(mode, read, hs, nh, B, T, x1, x2, w, mask, out_y, out_dx, out_dw, out_k, out_s,
+                                       out_kernels);
+      case GINN_HIP_F16:
+        return permuted_products<Half>(mode, read, hs, nh, B, T, x1, x2, w, mask, out_y, out_dx, out_dw, out_k, out_s,
+                                       out_kernels);
+      case GINN_HIP_BF16:
+        return permuted_products<BFloat16>(mode, read, hs, nh, B, T, x1, x2, w, mask, out_y, out_dx, out_dw, out_k,
+                                           out_s, out_kernels);
+    }
+    g_error = "unknown dtype";
+    return 1;
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return 2;
+  }
+}
+
 int shim_shared_weight_graph(int mode, int d, const float* w, const float* v, const float* x1, const float* x2,
                              float* out_loss, float* out_dw, float* out_dv, long* out_beside) {
   try {

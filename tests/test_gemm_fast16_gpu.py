@@ -272,6 +272,58 @@ def test_small_slice_batches(dev, dt, op_a, op_b, m, n, k, batch):
 
 
 @pytest.mark.parametrize("dt", [capi.F16, capi.BF16, capi.F32])
+@pytest.mark.parametrize("hs,nh,B,T", [(64, 12, 8, 512), (64, 3, 4, 128), (32, 5, 3, 72)])
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_two_level_batches_on_the_attention_layout(dev, dt, hs, nh, B, T, beta):
+    """ginn_hip_gemm_strided_batched2 on operands as the projections of an attention layer leave them: K, Q, V
+    are [hs nh x B T] matrices (element (e, h, b, t) at e + hs (h + nh (b + B t))), slice z = b + B h of each is
+    the [hs x T] matrix with leading dimension hs nh B at 64 h + hs nh b -- two levels of strides.  Scores
+    S = K^T Q (TN, [T x T] slices, contiguous), output Y = V P written back into the [hs nh x B T] layout, and
+    the gradient dK^T = Q dS^T (NT) written strided as well.  16-bit 64-row slices take the small-slice kernel in
+    one launch; fp32 and the odd sizes run level by level on the other kernels; against numpy fp64."""
+    from gpu_util import round_to, torch_dtype
+    torch = dev.torch
+    rng = np.random.default_rng(hs + nh + B + T)
+    C_ = hs * nh
+
+    def proj():
+        return round_to(rng.standard_normal((hs, nh, B, T)) / np.sqrt(hs), dt)
+
+    K, Q, V = proj(), proj(), proj()
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a.reshape(-1, order="F"))).to("cuda").to(torch_dtype(dt))
+    dK_, dQ_, dV_ = up(K), up(Q), up(V)
+    ld, s_b, s_h, batch = C_ * B, C_, hs, B * nh
+    call = lambda *a: dev.lib.call("ginn_hip_gemm_strided_batched2", dev.ctx, dt, *a)
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    # scores: [T x T] per slice, contiguous slices numbered z = b + B h
+    S0 = round_to(rng.standard_normal((T, T, B, nh)), dt)
+    dS = up(S0)
+    call(1, 0, T, T, hs, ptr(dK_), ld, s_b, s_h, ptr(dQ_), ld, s_b, s_h, beta, ptr(dS), T, T * T, T * T * B, B, nh)
+    dev.sync()
+    got = dS.double().cpu().numpy().reshape((T, T, B, nh), order="F")
+    want = np.einsum("ehbt,ehbu->tubh", K.astype(np.float64), Q.astype(np.float64)) + beta * S0
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) <= _bound(dt)
+    # output: Y[e, h, b, t] = sum_u V[e, h, b, u] P[u, t, b, h], written in the projections' layout
+    P = round_to(rng.uniform(0, 2.0 / T, (T, T, B, nh)), dt)
+    Y0 = proj()
+    dP, dY = up(P), up(Y0)
+    call(0, 0, hs, T, T, ptr(dV_), ld, s_b, s_h, ptr(dP), T, T * T, T * T * B, beta, ptr(dY), ld, s_b, s_h, B, nh)
+    dev.sync()
+    got = dY.double().cpu().numpy().reshape((hs, nh, B, T), order="F")
+    want = np.einsum("ehbu,utbh->ehbt", V.astype(np.float64), P.astype(np.float64)) + beta * Y0
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) <= _bound(dt)
+    # gradient of K through its transposed view: dKview[e, h, b, t] = sum_u Q[e, h, b, u] G[t, u, b, h]
+    G = round_to(rng.standard_normal((T, T, B, nh)) / np.sqrt(T), dt)
+    D0 = proj()
+    dG, dD = up(G), up(D0)
+    call(0, 1, hs, T, T, ptr(dQ_), ld, s_b, s_h, ptr(dG), T, T * T, T * T * B, beta, ptr(dD), ld, s_b, s_h, B, nh)
+    dev.sync()
+    got = dD.double().cpu().numpy().reshape((hs, nh, B, T), order="F")
+    want = np.einsum("ehbu,tubh->ehbt", Q.astype(np.float64), G.astype(np.float64)) + beta * D0
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) <= _bound(dt)
+
+
+@pytest.mark.parametrize("dt", [capi.F16, capi.BF16, capi.F32])
 @pytest.mark.parametrize("op_a,op_b,m,n,k", [(0, 0, 512, 512, 64), (0, 0, 256, 256, 64), (0, 1, 256, 256, 64),
                                              (1, 0, 256, 128, 256), (0, 0, 128, 512, 512), (0, 0, 256, 64, 256),
                                              (0, 1, 256, 64, 256), (1, 0, 64, 256, 256), (0, 0, 64, 512, 512),

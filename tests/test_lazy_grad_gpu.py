@@ -206,3 +206,65 @@ def test_a_skipped_backward_does_not_leak_into_the_next_pass(shim):
     assert np.abs(out[6:]).max() > 0
     assert (out[6:].reshape(3, 2, order="F")[mask == 0] == 0).all()  # masked entries pass no gradient
     np.testing.assert_array_equal(out[:6], out[6:])
+
+
+@pytest.mark.parametrize("dt", [capi.F32, capi.BF16, capi.F16])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("read", [0, 1])
+@pytest.mark.parametrize("hs,nh,B,T", [(64, 4, 8, 64), (16, 2, 3, 24), (64, 8, 16, 256)])
+def test_batched_products_on_permuted_views(shim, dt, mode, read, hs, nh, B, T):
+    """Permute nodes between projections and batched products (the heads of an attention layer,
+    examples/min-gpt.cu.cpp:117-135) copy nothing: BatchedProd reads the slices where the projection wrote
+    them, writes its result where the next node reads it, and the gradients take the same ways back
+    (ginn_amd/ginn/node/slices.h).  Values and gradients against numpy fp64, node by node and through the level
+    executor, frozen and recorded; the input changes between the passes, so a frozen pass that replayed a
+    value instead of computing it would differ; with `read` the postponed values are asked for mid-pass.
+    The 64-row heads in 16 bit take the one-launch two-level kernel, the others run level by level."""
+    from gpu_util import TOL, round_to
+    if T == 256 and (mode != 3 or read or dt == capi.F32):
+        pytest.skip("the large case checks the one-launch kernel and the launch count of a recorded pass")
+    C, N = hs * nh, B * T
+    rng = np.random.default_rng(hs + T + mode)
+    x1 = np.asfortranarray(round_to(rng.uniform(-1, 1, (C, N)), dt))
+    x2 = np.asfortranarray(round_to(rng.uniform(-1, 1, (C, N)), dt))
+    W = [np.asfortranarray(round_to(rng.uniform(-1, 1, (C, C)) / math.sqrt(C), dt)) for _ in range(3)]
+    mask = np.asfortranarray(round_to(rng.uniform(-1, 1, (C, N)), dt))
+    y = np.zeros((C, N), np.float32, order="F")
+    dx = np.zeros((C, N), np.float32, order="F")
+    dW = [np.zeros((C, C), np.float32, order="F") for _ in range(3)]
+    k_out = np.zeros((T, hs, B, nh), np.float32, order="F")
+    s_out = np.zeros((T, T, B, nh), np.float32, order="F")
+    kernels = ctypes.c_long(-1)
+    rc = shim.shim_permuted_products(dt, mode, read, hs, nh, B, T, fptr(x1), fptr(x2),
+                                     (ctypes.POINTER(ctypes.c_float) * 3)(*[fptr(w) for w in W]), fptr(mask), fptr(y),
+                                     fptr(dx), (ctypes.POINTER(ctypes.c_float) * 3)(*[fptr(g) for g in dW]),
+                                     fptr(k_out), fptr(s_out), ctypes.byref(kernels))
+    assert rc == 0, shim.lazy_last_error().decode()
+    # numpy fp64 on x2: projections [hs, nh, B, T]; s[t, u, b, h] = sum_e K[e,h,b,t] Q[e,h,b,u]; y = V s
+    X, Wk, Wq, Wv, M = (a.astype(np.float64) for a in (x2, W[0], W[1], W[2], mask))
+    heads = lambda P: P.reshape((hs, nh, B, T), order="F")
+    K, Q, V = heads(Wk @ X), heads(Wq @ X), heads(Wv @ X)
+    S = np.einsum("ehbt,ehbu->tubh", K, Q)
+    Y = np.einsum("ehbt,tubh->ehbu", V, S)
+    dY = heads(M)
+    dV = np.einsum("ehbu,tubh->ehbt", dY, S)
+    dS = np.einsum("ehbt,ehbu->tubh", V, dY)
+    dK = np.einsum("tubh,ehbu->ehbt", dS, Q)
+    dQ = np.einsum("tubh,ehbt->ehbu", dS, K)
+    flat = lambda P: P.reshape((C, N), order="F")
+    want_dW = [flat(dK) @ X.T, flat(dQ) @ X.T, flat(dV) @ X.T]
+    want_dx = Wk.T @ flat(dK) + Wq.T @ flat(dQ) + Wv.T @ flat(dV)
+    tol = 4 * TOL[dt]
+    assert rel_fro(y, flat(Y)) <= tol
+    assert rel_fro(dx, want_dx) <= tol
+    for got, want in zip(dW, want_dW):
+        assert rel_fro(got, want) <= tol
+    if read:
+        assert rel_fro(k_out, np.transpose(K, (3, 0, 2, 1))) <= tol
+        assert rel_fro(s_out, S) <= tol
+    if mode == 3 and T == 256:
+        # three projections, two batched products, the element-wise product and the sum forward; backward
+        # the broadcast, the product with the mask, four batched products and six projections' products
+        # (those of the weights with their split-K folds) plus the fills of reset_grad: 28 launches, none of
+        # them a copy for one of the four Permute nodes (8 more, forward and backward, with the copies)
+        assert 0 < kernels.value <= 30, kernels.value
