@@ -628,7 +628,27 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
   constexpr int kRowChunks = 4 * FM;
   constexpr int kColsPerIter = 64 / kRowChunks;
   const int sub = lane / kRowChunks, chunk = lane % kRowChunks;
-  if (EPI == kPlain) {
+  // A bias alone (no old C, no activation, no kept pre-activation) is added to the accumulators where they
+  // are -- a lane holds four consecutive rows per group -- and the tile leaves through the plain path: the
+  // same single rounding of acc + bias without the fp32 staging of the general path.
+  const bool bias_only = EPI == kGeneral && p.beta == 0.f && p.act == GINN_HIP_ACT_IDENTITY && p.pre == nullptr;
+  if (bias_only && p.bias) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int r = m0 + wm + i * 32 + 8 * b + 4 * lhi;
+        u16x4 bv = {0, 0, 0, 0};
+        if (r < p.m) bv = *reinterpret_cast<const u16x4*>(static_cast<const uint16_t*>(p.bias) + r);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float add = to_float<T>(bv[e]);
+#pragma unroll
+          for (int j = 0; j < FN; ++j) acc[i][j][4 * b + e] += add;
+        }
+      }
+  }
+  if (EPI == kPlain || bias_only) {
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
