@@ -299,9 +299,11 @@ def bench_lstm(iters, cpu, mode=7, gather=False):
     return r
 
 
-def bench_attention(h, steps, warmup, cpu):
+def bench_attention(h, steps, warmup, cpu, store_floor=False):
     """BatchedProd attention products, fp16: batch 128, QK^T [256x64][64x256] and PV [256x256][256x64],
-    forward and both backward products of each."""
+    forward and both backward products of each.  store_floor: one more line, a plain fill of the 16.8 MB
+    that the two products with a [256 x 256] result store -- what writing those bytes costs with no operand
+    read and no arithmetic, launch included."""
     import numpy as np
     t = h.torch
     cases = [("QK^T fwd  NN", 0, 0, 256, 256, 64), ("QK^T dK   NT", 0, 1, 256, 64, 256),
@@ -347,6 +349,22 @@ def bench_attention(h, steps, warmup, cpu):
             r["cpu_ms"] = round(_cpu_timed(lambda: cgemm.bgemm(a, b, op_a=op_a, op_b=op_b, kind="f32", threads=1)), 2)
             r["cpu"] = "oracle_bgemm_f32, 1 thread"
         out.append(r)
+    if store_floor:
+        n = batch * 256 * 256
+        buf = t.empty(n, device="cuda", dtype=t.float16)
+        ms = c_float(0)
+        for _ in range(2):
+            for i in range(warmup + steps):
+                if i == warmup:
+                    h.lib.call("ginn_hip_event_record", h.ctx, 0)
+                h.lib.call("ginn_hip_fill", h.ctx, DT["f16"], c_void_p(buf.data_ptr()), n, c_float(1.0))
+            h.lib.call("ginn_hip_event_record", h.ctx, 1)
+            h.lib.call("ginn_hip_sync", h.ctx)
+            h.lib.call("ginn_hip_event_elapsed_ms", h.ctx, 0, 1, byref(ms))
+        ms = ms.value / steps
+        out.append({"config": "fill of 16.8 MB fp16 (the bytes a [256 x 256] x 128 result stores; calls issued from "
+                              "Python, see the kernel trace for the kernel alone)", "gpu_ms": round(ms, 5),
+                    "gbs": round(2.0 * n / ms / 1e6, 1), "frac_hbm": round(2.0 * n / ms / 1e6 / PEAK_HBM_GBS, 4)})
     return out
 
 
@@ -641,7 +659,7 @@ def main():
             out.append(bench_lstm(max(1, iters // 20), False, mode=1))
             out.append(bench_lstm(max(1, iters // 20), False, mode=0))
         if a.workload in ("configs", "attention"):
-            out.extend(bench_attention(h, iters, a.warmup, cpu))
+            out.extend(bench_attention(h, iters, a.warmup, cpu, store_floor=a.workload == "attention"))
         if a.workload in ("configs", "update"):
             out.extend(bench_update(h, iters, a.warmup, cpu))
         if a.workload in ("configs", "gpt"):
