@@ -296,6 +296,20 @@ def bench_lstm(iters, cpu, mode=7, gather=False):
         xl = [np.asfortranarray(xs[:, offs[s]:offs[s + 1]]) for s in range(nseq)]
         r["cpu_ms"] = round(_cpu_timed(lambda: N.lstm_backward(W, b, xl, mask)), 2)
         r["cpu"] = "oracle (numpy fp32, sequences batched per step), 1 thread"
+        # The same graph with its nodes on cpu(): node by node through the host layer's own loops (no Autobatch,
+        # one Affine per sequence step, as the reference runs it on its CPU device), one pass.
+        ex.scenario_set_device(1)
+        try:
+            cms = ctypes.c_float(0)
+            rc = ex.scenario_lstm(0, nseq, (ctypes.c_int * nseq)(*lens), E, H, _fp(W), _fp(b), _fp(xs), _fp(mask),
+                                  1, _fp(out_h), _fp(loss), _fp(dW), _fp(db), _fp(dxs), ctypes.byref(cms),
+                                  ctypes.byref(nodes), ctypes.byref(prods), ctypes.byref(launches), None)
+        finally:
+            ex.scenario_set_device(0)
+        if rc:
+            raise SystemExit(ex.scenario_last_error().decode())
+        r["cpu_nodes_ms"] = round(cms.value, 1)
+        r["cpu_nodes"] = "the same graph on cpu(): host layer nodes, one Affine per sequence step, 1 thread"
     return r
 
 
@@ -510,6 +524,8 @@ def bench_gpt(iters, cpu, dtype="bf16", executor=6, train=None):
                    f"(block + final LayerNorm + head + loss), executor={executor}",
          "gpu_ms": round(ms.value, 3), "tflops": round(3 * fwd / ms.value / 1e9, 1), "graph_nodes": nodes.value,
          "loss": round(float(loss[0]), 4)}
+    if executor & 8:
+        r["kernels_per_pass"] = int(ex.scenario_recorded_kernels())
     if cpu:
         from oracle import nodes as N
         p = N.GptBlockParams(**params)
@@ -570,6 +586,7 @@ def other_configs(h, cpu):
     out["gpt_ms"], out["gpt_tflops"] = g["gpu_ms"], g["tflops"]
     if cpu:
         out["gpt_cpu_ms"] = g["cpu_ms"]
+    out["gpt_kernels_per_pass"] = bench_gpt(2, False, executor=14)["kernels_per_pass"]
     r = bench_mlp(100, cpu, executor=6)
     out["mlp_ms"], out["mlp_gbs"] = r["gpu_ms"], r["gbs"]
     if cpu:
@@ -581,6 +598,7 @@ def other_configs(h, cpu):
     out["lstm_table_launches_per_pass"] = r["table_launches_per_pass"]
     if cpu:
         out["lstm_cpu_ms"] = r["cpu_ms"]
+        out["lstm_cpu_nodes_ms"] = r["cpu_nodes_ms"]
     out["lstm_kernels_per_pass"] = bench_lstm(2, False, mode=31, gather=True)["kernels_per_pass"]
     out["attention"] = {r["config"].split("batch 128 ")[1]: {"us": round(r["gpu_ms"] * 1e3, 2), "gbs": r["gbs"],
                                                              "frac_hbm": r["frac_hbm"], "tflops": r["tflops"]}
@@ -604,8 +622,8 @@ def other_configs(h, cpu):
                    "autobatched LSTM fp32 256 seqs; gbs = algorithmic bytes of the pass's products per second; "
                    "kernels_per_pass = kernel nodes of the pass recorded as a device graph; attention = fp16 batch 128 "
                    "products, skinny = M = K = 4096 NN with the split-K fold included, against 8 TB/s; squares "
-                   "against 2.5 PFLOP/s; cpu = numpy fp32 oracle on 1 thread; mlp_cpu_nodes_ms = the same MLP graph with "
-                   "its nodes on cpu() (the host layer's own fp32 loops, 1 thread)")
+                   "against 2.5 PFLOP/s; cpu = numpy fp32 oracle on 1 thread; mlp_cpu_nodes_ms / lstm_cpu_nodes_ms = the same "
+                   "graph with its nodes on cpu() (the host layer's own fp32 loops, node by node, 1 thread)")
     return out
 
 

@@ -27,7 +27,7 @@ using namespace ginn;
 namespace {
 
 thread_local std::string g_error;
-// scenario_set_device(1): the MLP scenario keeps its graph on cpu() and runs through the host layer's own
+// scenario_set_device(1): the scenarios keep their graphs on cpu() and run through the host layer's own
 // loops (ginn/cpu_ops.h), node by node -- the same graph code as on the device, as a host baseline.
 bool g_on_cpu = false;
 DevPtr place() { return g_on_cpu ? DevPtr(cpu()) : DevPtr(gpu()); }
@@ -353,8 +353,8 @@ int lstm(int mode, int nseq, const int* lens, int E, int H, const float* W, cons
   std::vector<NodePtr<Real>> finals;
   Size col = 0;
   for (int s = 0; s < nseq; ++s) {
-    NodePtr<Real> h = Zero<Real>(gpu(), Shape{H, 1});
-    NodePtr<Real> c = Zero<Real>(gpu(), Shape{H, 1});
+    NodePtr<Real> h = Zero<Real>(place(), Shape{H, 1});
+    NodePtr<Real> c = Zero<Real>(place(), Shape{H, 1});
     for (int t = 0; t < lens[s]; ++t, ++col) {
       auto x = Slice(NodePtr<Real>(X), Shape{0, col}, Shape{E, 1});
       auto z = Affine(Wn, Cat(NodePtr<Real>(x), h), bn);
@@ -437,7 +437,7 @@ int gpt_layer(int C, int nh, int B, int T, int V, const float* x, const int* tar
   auto X = data_from<S>({C, B, T}, x, true);
   auto Y = Data<Int>(cpu(), Shape{B * T});
   for (int i = 0; i < B * T; ++i) Y->value().v()[i] = targets[i];
-  Y->move_to(gpu());
+  Y->move_to(place());
   Y->set_has_grad(false);
 
   auto ln = [&](const NodePtr<S>& v, int g, int b) -> NodePtr<S> {
@@ -453,7 +453,7 @@ int gpt_layer(int C, int nh, int B, int T, int V, const float* x, const int* tar
   auto q = rearrange(Affine(w[Wq], a1, w[bq]), {0, 3, 2, 1});  // hs, T, B, nh
   auto v = rearrange(Affine(w[Wv], a1, w[bv]), {0, 3, 2, 1});  // hs, T, B, nh
   NodePtr<S> att = InPlaceProdScalar(NodePtr<S>(BatchedProd(k, q)), 1.f / std::sqrt(static_cast<float>(hs)));
-  NodePtr<S> mask = Reshape(NodePtr<S>(UpperTri<S>(gpu(), static_cast<Size>(T))), Shape{T, T, 1, 1});
+  NodePtr<S> mask = Reshape(NodePtr<S>(UpperTri<S>(place(), static_cast<Size>(T))), Shape{T, T, 1, 1});
   att = InPlaceMask(att, mask, -std::numeric_limits<float>::infinity());
   att = Softmax(att);
   NodePtr<S> y = BatchedProd(v, att);  // hs, T, B, nh
@@ -603,7 +603,8 @@ int scenario_lstm(int mode, int nseq, const int* lens, int E, int H, const float
 // node), 2 = level executor, 6 = level executor frozen after its first pass, 14 = the frozen pass as a
 // recorded device graph.
 void scenario_set_executor(int mode) { g_exec_mode = mode; }
-// 1: scenario_mlp builds and runs its graph on cpu() (host loops, node by node); 0: on the HIP device.
+// 1: scenario_mlp, scenario_lstm (mode 0) and scenario_gpt_layer (executor 0) build and run their graphs on
+// cpu() (the host layer's own loops, node by node); 0: on the HIP device.
 void scenario_set_device(int on_cpu) { g_on_cpu = on_cpu != 0; }
 
 // Training rule of scenario_gpt_layer from now on: -1 = none (forward + backward only), 0 = Sgd, 1 = Adam;

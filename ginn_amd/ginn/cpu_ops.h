@@ -246,6 +246,124 @@ void pick_nls_backward(int rows, int cols, const S* x, const int* index, const S
   }
 }
 
+// dst (+)= src over a [rows x cols] window with leading dimensions lds / ldd (Slice, Cat, RowwiseCat, Chip).
+template <typename S>
+void copy_2d(Size rows, Size cols, const S* src, Size lds, S* dst, Size ldd, bool accumulate) {
+  for (Size c = 0; c < cols; ++c)
+    for (Size r = 0; r < rows; ++r) {
+      if constexpr (std::is_arithmetic_v<S> && !std::is_floating_point_v<S>) {
+        dst[c * ldd + r] = src[c * lds + r];  // integer tensors are only moved
+      } else {
+        const float v = get(src, c * lds + r);
+        put(dst, c * ldd + r, accumulate ? get(dst, c * ldd + r) + v : v);
+      }
+    }
+}
+
+// dst[permuted index] (+)= src[index]: dst has extents dims[perm[0]], dims[perm[1]], ... (PermuteNode).
+template <typename S>
+void permute(const std::vector<Size>& dims, const std::vector<Size>& perm, const S* src, S* dst, bool accumulate) {
+  const size_t rank = dims.size();
+  std::vector<Size> src_stride(rank), dst_stride_of_src_axis(rank), idx(rank, 0);
+  Size run = 1, total = 1;
+  for (size_t i = 0; i < rank; ++i) {
+    src_stride[i] = run;
+    run *= dims[i];
+  }
+  total = run;
+  run = 1;
+  for (size_t j = 0; j < rank; ++j) {  // axis j of dst runs along axis perm[j] of src
+    dst_stride_of_src_axis[static_cast<size_t>(perm[j])] = run;
+    run *= dims[static_cast<size_t>(perm[j])];
+  }
+  for (Size lin = 0; lin < total; ++lin) {
+    Size d = 0;
+    for (size_t i = 0; i < rank; ++i) d += idx[i] * dst_stride_of_src_axis[i];
+    const float v = get(src, lin);
+    put(dst, d, accumulate ? get(dst, d) + v : v);
+    for (size_t i = 0; i < rank; ++i) {  // next index of src, first axis fastest
+      if (++idx[i] < dims[i]) break;
+      idx[i] = 0;
+    }
+  }
+}
+
+// LayerNorm per column (ginn/node/layernorm.h:31-74): y = (x - mean) / std, std = sqrt(mean((x - mean)^2) + eps);
+// dx (+)= (dy - mean(dy) - y <dy, y> / rows) / std.
+template <typename S>
+void layernorm_forward(int rows, int cols, const S* x, float eps, S* y, float* std_out) {
+  for (int c = 0; c < cols; ++c) {
+    const size_t o = static_cast<size_t>(c) * rows;
+    double mean = 0., var = 0.;
+    for (int r = 0; r < rows; ++r) mean += get(x, o + r);
+    mean /= rows;
+    for (int r = 0; r < rows; ++r) {
+      const double d = get(x, o + r) - mean;
+      var += d * d;
+    }
+    const float sd = std::sqrt(static_cast<float>(var / rows) + eps);
+    std_out[c] = sd;
+    for (int r = 0; r < rows; ++r) put(y, o + r, (get(x, o + r) - static_cast<float>(mean)) / sd);
+  }
+}
+template <typename S>
+void layernorm_backward(int rows, int cols, const S* dy, const S* y, const float* std_in, S* dx, bool accumulate) {
+  for (int c = 0; c < cols; ++c) {
+    const size_t o = static_cast<size_t>(c) * rows;
+    double sum = 0., dot = 0.;
+    for (int r = 0; r < rows; ++r) {
+      sum += get(dy, o + r);
+      dot += static_cast<double>(get(dy, o + r)) * get(y, o + r);
+    }
+    const float m = static_cast<float>(sum / rows), d = static_cast<float>(dot / rows);
+    for (int r = 0; r < rows; ++r) {
+      const float v = (get(dy, o + r) - m - get(y, o + r) * d) / std_in[c];
+      put(dx, o + r, accumulate ? get(dx, o + r) + v : v);
+    }
+  }
+}
+
+// CwiseProdAdd (ginn/node/common.h:251-316): y = a (*) (b + bias) + c, b and c per row when `broadcast`.
+template <typename S>
+void cwise_prod_add_forward(int rows, int cols, const S* a, const S* b, const S* c, float bias, bool broadcast, S* y) {
+  const size_t n = static_cast<size_t>(rows) * cols;
+  for (size_t i = 0; i < n; ++i) {
+    const size_t j = broadcast ? i % rows : i;
+    put(y, i, get(a, i) * (get(b, j) + bias) + get(c, j));
+  }
+}
+// da (+)= dy (*) (b + bias); db += dy (*) a; dc += dy (row sums when `broadcast`).
+template <typename S>
+void cwise_prod_add_backward(int rows, int cols, const S* dy, const S* a, const S* b, float bias, bool broadcast, S* da,
+                             bool da_accumulate, S* db, S* dc) {
+  const size_t n = static_cast<size_t>(rows) * cols, nb = broadcast ? static_cast<size_t>(rows) : n;
+  std::vector<float> sb, sc;
+  if (db) sb.assign(nb, 0.f);
+  if (dc) sc.assign(nb, 0.f);
+  for (size_t i = 0; i < n; ++i) {
+    const size_t j = broadcast ? i % rows : i;
+    const float g = get(dy, i);
+    if (da) {
+      const float v = g * (get(b, j) + bias);
+      put(da, i, da_accumulate ? get(da, i) + v : v);
+    }
+    if (db) sb[j] += g * get(a, i);
+    if (dc) sc[j] += g;
+  }
+  for (size_t j = 0; j < nb; ++j) {
+    if (db) put(db, j, get(db, j) + sb[j]);
+    if (dc) put(dc, j, get(dc, j) + sc[j]);
+  }
+}
+
+// x viewed as [mask_size x batch]: entries whose mask value is 0 become `value` (InPlaceMask).
+template <typename S>
+void mask_fill(size_t mask_size, size_t batch, const S* mask, float value, S* x) {
+  for (size_t z = 0; z < batch; ++z)
+    for (size_t i = 0; i < mask_size; ++i)
+      if (get(mask, i) == 0.f) put(x, z * mask_size + i, value);
+}
+
 }  // namespace host
 }  // namespace ginn
 

@@ -242,7 +242,6 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
   float multiplier_bias_;
 
   void forward_() override {
-    internal::require_gpu(this->dev(), "CwiseProdAdd");
     // shape(), not value(): a LayerNorm in front that has not run yet stays so
     const Shape s0 = a_->shape(), s1 = b_->value().shape(), s2 = c_->value().shape();
     if (s0 == s1 && s1 == s2) {
@@ -254,6 +253,15 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
       GINN_THROW("Unexpected shapes for CwiseProdAdd!");
     }
     value().resize(s0);
+    if (this->dev()->kind() == CPU) {
+      if constexpr (is_floating_point_v<Scalar>) {
+        auto& a = a_->value();
+        return host::cwise_prod_add_forward<Scalar>(static_cast<int>(a.rows()), static_cast<int>(a.cols()), a.data(),
+                                                    b_->value().data(), c_->value().data(), multiplier_bias_,
+                                                    broadcast_, value().data());
+      }
+    }
+    internal::require_gpu(this->dev(), "CwiseProdAdd");
     // Right behind a LayerNorm whose kernel has not run yet: normalisation and
     // the gamma / beta step as one pass (same values).
     if (LayerNormNode<Scalar>* ln = broadcast_ ? layer_norm() : nullptr; ln && ln->pending_) {
@@ -273,6 +281,15 @@ class CwiseProdAddNode : public BaseDataNode<Scalar> {
   }
   void backward_() override {
     auto& a = a_->value();
+    if (this->dev()->kind() == CPU) {
+      if constexpr (is_floating_point_v<Scalar>) {
+        const bool fresh = a_->has_grad() && a_->take_lazy_zero();
+        return host::cwise_prod_add_backward<Scalar>(
+            static_cast<int>(a.rows()), static_cast<int>(a.cols()), grad().data(), a.data(), b_->value().data(),
+            multiplier_bias_, broadcast_, a_->has_grad() ? a_->grad().data() : nullptr, !fresh,
+            b_->has_grad() ? b_->grad().data() : nullptr, c_->has_grad() ? c_->grad().data() : nullptr);
+      }
+    }
     internal::PostponeFolds later(internal::ctx_of(a), *b_, *c_);  // scale / shift gradients: complete at the pass's end
     // A flagged gradient of a means: this node is its only user and overwrites.
     const bool fresh = a_->has_grad() && a_->take_lazy_zero();

@@ -25,12 +25,13 @@ class InPlaceProdScalarNode : public BaseDataNode<Scalar>, public PendingInPlace
   bool skip_backward_ = false;
 
   void scale(Tensor<Scalar>& t) const {
+    if (t.dev()->kind() == CPU)
+      return host::scale_shift<Scalar>(static_cast<size_t>(t.size()), val_, 0.f, t.data(), t.data(), false);
     internal::require_gpu(t.dev(), "InPlaceProdScalar");
     GINN_HIP_CALL(ginn_hip_scale_shift(internal::ctx_of(t), dtype_of<Scalar>(), static_cast<size_t>(t.size()), val_,
                                        0.f, t.data(), t.data(), 0));
   }
   void forward_() override {
-    internal::require_gpu(in_->dev(), "InPlaceProdScalar");
     pending_ = true;
     skip_backward_ = false;
   }
@@ -86,8 +87,11 @@ class InPlaceMaskNode : public BaseDataNode<Scalar>, public PendingInPlace {
   bool skip_backward_ = false;
 
   void fill(Tensor<Scalar>& t, float v) const {
-    internal::require_gpu(t.dev(), "InPlaceMask");
     const Size ms = mask_->value().size();
+    if (t.dev()->kind() == CPU)
+      return host::mask_fill<Scalar>(static_cast<size_t>(ms), static_cast<size_t>(t.size() / ms), mask_->value().data(),
+                                     v, t.data());
+    internal::require_gpu(t.dev(), "InPlaceMask");
     GINN_HIP_CALL(ginn_hip_mask_fill(internal::ctx_of(t), dtype_of<Scalar>(), static_cast<size_t>(ms),
                                      static_cast<size_t>(t.size() / ms), mask_->value().data(), v, t.data()));
   }
@@ -98,7 +102,6 @@ class InPlaceMaskNode : public BaseDataNode<Scalar>, public PendingInPlace {
     while (i < is.size() && ms[i] == is[i]) ++i;
     for (; i < is.size(); ++i) GINN_ASSERT(ms[i] == 1, "Unexpected mask shape!");
     GINN_ASSERT(mask_->value().size() > 0);
-    internal::require_gpu(in_->dev(), "InPlaceMask");
     pending_ = true;
     skip_backward_ = false;
   }

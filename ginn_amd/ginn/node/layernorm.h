@@ -35,12 +35,16 @@ class LayerNormNode : public BaseDataNode<Scalar>, public PostponedValue {
   void normalise() const {
     auto& x = in_->value();
     Tensor<Scalar>& y = may_postpone() ? raw_value() : const_cast<LayerNormNode*>(this)->value();
+    if (x.dev()->kind() == CPU) {
+      host::layernorm_forward<Scalar>(static_cast<int>(x.rows()), static_cast<int>(x.cols()), x.data(), eps_, y.data(),
+                                      const_cast<Tensor<float>&>(std_).data());
+      return;
+    }
     GINN_HIP_CALL(ginn_hip_layernorm_fwd(internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()),
                                          static_cast<int>(x.cols()), x.data(), eps_, y.data(),
                                          const_cast<Tensor<float>&>(std_).data()));
   }
   void forward_() override {
-    internal::require_gpu(in_->dev(), "LayerNorm");
     const Shape s = in_->shape();
     const Size rows = s.empty() ? 1 : s[0];
     std_.resize({1, rows > 0 ? Tensor<Scalar>::size(s) / rows : 0});
@@ -60,6 +64,11 @@ class LayerNormNode : public BaseDataNode<Scalar>, public PostponedValue {
     if (!in_->has_grad()) return;
     auto& y = value();
     const bool fresh = in_->take_lazy_zero();
+    if (y.dev()->kind() == CPU) {
+      host::layernorm_backward<Scalar>(static_cast<int>(y.rows()), static_cast<int>(y.cols()), grad().data(), y.data(),
+                                       std_.data(), in_->grad().data(), !fresh);
+      return;
+    }
     GINN_HIP_CALL((fresh ? ginn_hip_layernorm_bwd_assign : ginn_hip_layernorm_bwd)(
         internal::ctx_of(y), dtype_of<Scalar>(), static_cast<int>(y.rows()), static_cast<int>(y.cols()),
         grad().data(), y.data(), std_.data(), in_->grad().data()));

@@ -4,6 +4,7 @@
 #ifndef GINN_NODE_LAYOUT_H
 #define GINN_NODE_LAYOUT_H
 
+#include <ginn/cpu_ops.h>
 #include <ginn/node/data.h>
 #include <ginn/node/slices.h>
 #include <ginn/nonlin.h>
@@ -27,8 +28,12 @@ inline ginn_hip_dtype move_dtype_of() {
 template <typename Scalar>
 void copy_2d(Tensor<Scalar>& dst, Size dst_off, Size ldd, const Tensor<Scalar>& src, Size src_off, Size lds,
              Size rows, Size cols, bool accumulate) {
-  require_gpu(dst.dev(), "copy_2d");
   GINN_ASSERT(!accumulate || is_floating_point_v<Scalar>, "only floating-point tensors are added to");
+  if (dst.dev()->kind() == CPU) {
+    host::copy_2d<Scalar>(rows, cols, src.data() + src_off, lds, dst.data() + dst_off, ldd, accumulate);
+    return;
+  }
+  require_gpu(dst.dev(), "copy_2d");
   GINN_HIP_CALL(ginn_hip_copy_2d(ctx_of(dst), move_dtype_of<Scalar>(), static_cast<int>(rows), static_cast<int>(cols),
                                  src.data() + src_off, static_cast<int>(lds), dst.data() + dst_off,
                                  static_cast<int>(ldd), accumulate ? 1 : 0));
@@ -549,6 +554,10 @@ class PermuteNode : public BaseDataNode<Scalar>, public internal::SliceProvider<
 
   static void run(const Tensor<Scalar>& src, const Shape& src_shape, const Shape& perm, Tensor<Scalar>& dst,
                   bool accumulate) {
+    if (dst.dev()->kind() == CPU) {
+      if constexpr (is_floating_point_v<Scalar>)
+        return host::permute<Scalar>(src_shape, perm, src.data(), dst.data(), accumulate);
+    }
     internal::require_gpu(dst.dev(), "Permute");
     std::vector<long long> dims(src_shape.begin(), src_shape.end());
     std::vector<int> p(perm.begin(), perm.end());
@@ -830,9 +839,14 @@ class UpperTriNode : public BaseDataNode<Scalar> {
   DimPtr size_;
 
   void forward_() override {
-    internal::require_gpu(this->dev(), "UpperTri");
     const Size s = size_->value();
     value().resize(s, s);
+    if (this->dev()->kind() == CPU) {
+      for (Size c = 0; c < s; ++c)
+        for (Size r = 0; r < s; ++r) value().data()[c * s + r] = Scalar(r <= c ? 1.f : 0.f);
+      return;
+    }
+    internal::require_gpu(this->dev(), "UpperTri");
     GINN_HIP_CALL(ginn_hip_upper_tri(internal::ctx_of(value()), dtype_of<Scalar>(), static_cast<int>(s),
                                      value().data()));
   }

@@ -65,3 +65,42 @@ def test_mlp_configuration_on_cpu():
     assert rel_fro(nll, want_nll) <= 1e-4
     for got, ref in zip(dWs + dbs, list(want_dW) + list(want_db)):
         assert rel_fro(got, np.asarray(ref).reshape(got.shape)) <= 1e-4
+
+
+@pytest.fixture(scope="module")
+def cpu_scenarios():
+    """libginn_examples.so with its graphs placed on cpu() (scenario_set_device)."""
+    import test_scenarios_gpu as S
+    if not S.SHIM.exists():
+        pytest.fail(f"{S.SHIM} is missing: run __graft_entry__.build()")
+    capi.load()
+    lib = ctypes.CDLL(str(S.SHIM))
+    lib.scenario_last_error.restype = ctypes.c_char_p
+    lib.scenario_timed_fills.restype = ctypes.c_long
+    lib.scenario_set_executor(0)
+    lib.scenario_set_device(1)
+    yield lib
+    lib.scenario_set_device(0)
+
+
+@pytest.mark.parametrize("lens,E,H", [([3, 1, 4], 3, 2), ([5, 5, 5, 5], 8, 16), ([1], 4, 4),
+                                       ([7, 2, 9, 4, 4, 1, 12, 6], 128, 256)])
+def test_lstm_graph_on_cpu(cpu_scenarios, lens, E, H):
+    """The LSTM configuration's graph (Slice, Cat, Affine, gates, CwiseProd, Add, RowwiseCat, Sum) node by node
+    on cpu(): final states, loss and the gradients of W, b and the inputs against the oracle."""
+    import test_scenarios_gpu as S
+    got, want, stats = S.run_lstm(cpu_scenarios, 0, lens, E, H, seed=len(lens))
+    S.compare_lstm(got, want)
+    assert stats["prods"] == 0
+
+
+@pytest.mark.parametrize("C,nh,B,T,V", [(12, 3, 2, 5, 11), (64, 4, 3, 33, 50)])
+def test_gpt_layer_graph_on_cpu(cpu_scenarios, C, nh, B, T, V):
+    """The GPT layer's graph (LayerNorm + gamma / beta, projections, Reshape / Permute, BatchedProd, the in-place
+    scale and mask, Softmax, residuals, GELU MLP, head, PickNegLogSoftmax, Mean) node by node on cpu(): loss and
+    all 21 gradients against the oracle."""
+    import test_seqops_gpu as Q
+    loss, got, wloss, want, _ = Q.run_gpt(cpu_scenarios, capi.F32, C, nh, B, T, V, seed=C, wscale=0.2)
+    assert abs(loss - wloss) <= 1e-4 * abs(wloss)
+    errs = Q.grad_errors(got, want)
+    assert max(errs.values()) <= 1e-4, errs
