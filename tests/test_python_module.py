@@ -66,7 +66,7 @@ def test_nodes_on_cpu_compute_or_fail_loudly(ginn):
     p.forward()
     assert p.value.list() == [3.0, 7.0, 3.0, 7.0]
     with pytest.raises(RuntimeError, match="HIP device only"):
-        ginn.LayerNorm(x).forward()
+        ginn.Variance(x).forward()
 
 
 @pytest.mark.gpu
