@@ -162,9 +162,12 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 
-// EPI: false = plain store (beta == 0, no bias / activation / pre-activation),
-// staged through LDS for full-line stores; true = general epilogue.
-template <typename T, bool AKC, bool BKC, bool EPI>
+// EPI: 0 = plain store (beta == 0, no bias / activation / pre-activation), staged through LDS for
+// full-line stores; 1 = general epilogue; 2 = a bias alone: added to the accumulators where they are (a lane
+// holds four consecutive rows per group), then the plain store -- the same single rounding of acc + bias
+// as the general path, without its fp32 staging.  An instantiation of its own: as a run-time branch
+// inside the general one it made that kernel spill.
+template <typename T, bool AKC, bool BKC, int EPI>
 __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
   constexpr bool BF = std::is_same<T, BF16>::value;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -433,7 +436,23 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
   // column lane % 32.
   const int l32 = lane & 31, lhi = lane >> 5;
   uint16_t* C = p.C + bz * p.sc;
-  if (!EPI) {
+  if constexpr (EPI == 2) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int r = wm + i * 32 + 8 * b + 4 * lhi;
+        u16x4 bv = {0, 0, 0, 0};
+        if (r < m_valid) bv = *reinterpret_cast<const u16x4*>(p.bias + m0 + r);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float add = to_float<T>(bv[e]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[i][j][4 * b + e] += add;
+        }
+      }
+  }
+  if constexpr (EPI != 1) {
     // All LDS reads and direct loads of every wave ended before the last
     // barrier, so each wave may overwrite its own slice right away: write the
     // rounded tile column-major, read it back 16 bytes per lane, store full
@@ -555,15 +574,20 @@ __global__ __launch_bounds__(kThreads) void gemm_fast16_kernel(FastParams p) {
 }
 
 template <typename T, bool AKC, bool BKC>
-int launch_epi(ginn_hip_ctx* ctx, const FastParams& p, int batch, bool general) {
+int launch_epi(ginn_hip_ctx* ctx, const FastParams& p, int batch, int general) {
   const dim3 grid(p.tiles_m * p.tiles_n, batch);
-  if (general) {
-    auto fn = gemm_fast16_kernel<T, AKC, BKC, true>;
+  if (general == 2) {
+    auto fn = gemm_fast16_kernel<T, AKC, BKC, 2>;
+    static std::atomic<unsigned long long> lds_allowed{0};
+    GH_HIP(allow_dynamic_lds(lds_allowed, ctx->device, reinterpret_cast<const void*>(fn), kLdsBytes));
+    fn<<<grid, dim3(kThreads), kLdsBytes, ctx->stream>>>(p);
+  } else if (general == 1) {
+    auto fn = gemm_fast16_kernel<T, AKC, BKC, 1>;
     static std::atomic<unsigned long long> lds_allowed{0};
     GH_HIP(allow_dynamic_lds(lds_allowed, ctx->device, reinterpret_cast<const void*>(fn), kLdsBytes));
     fn<<<grid, dim3(kThreads), kLdsBytes, ctx->stream>>>(p);
   } else {
-    auto fn = gemm_fast16_kernel<T, AKC, BKC, false>;
+    auto fn = gemm_fast16_kernel<T, AKC, BKC, 0>;
     static std::atomic<unsigned long long> lds_allowed{0};
     GH_HIP(allow_dynamic_lds(lds_allowed, ctx->device, reinterpret_cast<const void*>(fn), kLdsBytes));
     fn<<<grid, dim3(kThreads), kLdsBytes, ctx->stream>>>(p);
@@ -573,7 +597,7 @@ int launch_epi(ginn_hip_ctx* ctx, const FastParams& p, int batch, bool general) 
 }
 
 template <typename T>
-int launch_layout(ginn_hip_ctx* ctx, const FastParams& p, int batch, bool akc, bool bkc, bool general) {
+int launch_layout(ginn_hip_ctx* ctx, const FastParams& p, int batch, bool akc, bool bkc, int general) {
   if (akc) {
     if (bkc) return launch_epi<T, true, true>(ctx, p, batch, general);
     return launch_epi<T, true, false>(ctx, p, batch, general);
@@ -637,7 +661,9 @@ int launch_gemm_fast16(ginn_hip_ctx* ctx, const GemmArgs& a) {
   // XCD-aware ordering needs the tile count to split evenly over the 8 XCDs.
   p.group = (tiles % 8 == 0) ? ((akc && bkc) ? 4 : 8) : 0;
   if (p.group > p.tiles_m) p.group = p.tiles_m;
-  const bool general = a.beta != 0.f || a.bias || a.pre || a.act != GINN_HIP_ACT_IDENTITY;
+  // 0 = plain, 1 = general, 2 = a bias alone (see the kernel)
+  const bool bias_only = a.bias && a.beta == 0.f && !a.pre && a.act == GINN_HIP_ACT_IDENTITY;
+  const int general = bias_only ? 2 : (a.beta != 0.f || a.bias || a.pre || a.act != GINN_HIP_ACT_IDENTITY) ? 1 : 0;
   if (a.dtype == GINN_HIP_F16) return launch_layout<F16>(ctx, p, a.batch, akc, bkc, general);
   return launch_layout<BF16>(ctx, p, a.batch, akc, bkc, general);
 }
