@@ -52,6 +52,7 @@ def parse_args():
                         "configs (MLP, autobatched LSTM, attention products, GPT layer: GPU time with the CPU "
                         "oracle beside) | mlp | lstm | attention | gpt | update (one of those alone, for profiling) | "
                         "ragged (products whose extents are no multiples of the tiles) | "
+                        "skinny (narrow right-hand sides against the HBM roofline) | "
                         "copy (a plain copy kernel of known size, to calibrate the HBM counters)")
     p.add_argument("--dtype", default="f16", choices=list(DT))
     p.add_argument("--layout", default="NN", choices=["NN", "NT", "TN"])
@@ -429,6 +430,23 @@ def bench_ragged(h, steps, warmup):
     return out
 
 
+def bench_skinny(h, steps, warmup):
+    """NN products with a narrow right-hand side, against the HBM roofline (A is read once): the skinny
+    shapes of the GEMM sweep (M = K = 4096, N = 1, 16, 64) and tall products over a smaller A, which run as
+    one launch (16-row strips over all of K) instead of a split of K plus a fold."""
+    cases = [(dt, 4096, n, 4096) for dt in ("f32", "f16", "bf16") for n in (1, 16, 64)]
+    cases += [("f16", 4096, 1, 1024), ("f16", 4096, 16, 1024), ("f16", 4096, 16, 2048), ("f16", 2048, 4, 2048),
+              ("f16", 2048, 1, 4096), ("f32", 4096, 16, 1024), ("f32", 4096, 16, 2048)]
+    time_product(h, "f16", "NN", 8192, 8192, 8192, 100, 100)  # untimed: lets the clocks settle
+    out = []
+    for dt, m, n, k in cases:
+        ms = time_product(h, dt, "NN", m, n, k, steps, warmup)
+        by = ESIZE[dt] * (m * k + k * n + m * n)
+        out.append({"config": f"{dt} NN {m}x{n}x{k}", "us": round(ms * 1e3, 2), "gbs": round(by / ms / 1e6, 1),
+                    "frac_hbm": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)})
+    return out
+
+
 def bench_update(h, steps, warmup, cpu):
     """One Adam / SGD step (ginn/update/update.h:54-133) over the weights of the GPT configuration (one
     decoder layer + vocabulary head, d 768, MLP 3072, vocab 8192: 13.4 M parameters in 14 tensors) in one
@@ -653,6 +671,11 @@ def main():
 
     if a.workload == "ragged":
         for r in bench_ragged(h, max(1, a.steps), a.warmup):
+            print(json.dumps(r), flush=True)
+        return
+
+    if a.workload == "skinny":
+        for r in bench_skinny(h, max(1, a.steps), a.warmup):
             print(json.dumps(r), flush=True)
         return
 
