@@ -52,7 +52,23 @@ static __device__ __attribute__((aligned(16))) const unsigned int kZeroChunk[4] 
 
 constexpr int kRowBytes = 128;  // bytes of one K tile along K: 64 16-bit or 32 fp32 values
 constexpr int kThreads = 512;   // 8 waves
-constexpr int kStages = 4;
+// LDS stages per tile shape.  The loads of a workgroup's next stages are all it has in flight.  Measured (bf16,
+// one MI355X, stages 4 / deeper): 64 x 64 tiles (16 KiB stages) 768 x 768 x 4096 17.2 / 15.9-16.0 us with 6 or 8
+// stages, 1024^3 and 1000^3 level; 128 x 128 tiles (32 KiB) get SLOWER with a fifth stage (768 x 4096 x 3072 TN
+// 24.5 -> 27.7 us, K = 8192 57.7 -> 63.3 us, fp32 2048^3 130 -> 136 us: their K loop is not waiting for latency) and
+// 128 x 64 tiles do not care (6 against 4 stages within 1 %).  GPT layer: 380 -> 384 TFLOP/s with 8 / 4 / 4.
+#ifndef GH_MID_STAGES_11
+#define GH_MID_STAGES_11 8
+#endif
+#ifndef GH_MID_STAGES_21
+#define GH_MID_STAGES_21 4
+#endif
+#ifndef GH_MID_STAGES_22
+#define GH_MID_STAGES_22 4
+#endif
+constexpr int stages_for(int fm, int fn) {
+  return fm + fn == 2 ? GH_MID_STAGES_11 : (fm + fn == 3 ? GH_MID_STAGES_21 : GH_MID_STAGES_22);
+}
 
 enum Epilogue { kPlain = 0, kGeneral = 1, kPartial = 2 };
 
@@ -62,7 +78,10 @@ struct Geo {
   static constexpr int kTileA = BM * kRowBytes;       // bytes of one A tile
   static constexpr int kTileB = BN * kRowBytes;
   static constexpr int kStageBytes = kTileA + kTileB;
+  static constexpr int kStages = stages_for(FM, FN);
+  static_assert(kStages >= 3 && kStages <= 8, "pipeline depth");
   static constexpr int kLdsBytes = kStages * kStageBytes;
+  static_assert(kLdsBytes <= 160 * 1024, "the stages must fit the LDS of a CU");
   // Epilogue staging inside the first two stages, per wave:
   //   plain: 32 FN columns x 32 FM halfs, column stride 64 FM + 16 bytes;
   //   general: 32 columns x 32 FM floats per pass, column stride 128 FM + 16 bytes.
@@ -207,6 +226,15 @@ __device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
   }
 }
 
+// f(R) for R = N, N - 1, ..., 1 as compile-time constants.
+template <int N, typename F>
+__device__ __forceinline__ void tail_tiles(F&& f) {
+  if constexpr (N >= 1) {
+    f(std::integral_constant<int, N>{});
+    tail_tiles<N - 1>(f);
+  }
+}
+
 // 8 waves: waves 4 .. 7 own the same output quadrants as waves 0 .. 3 but take
 // sub-steps 2, 3 of every K tile (waves 0 .. 3: sub-steps 0, 1) and hand their
 // sums over through LDS at the end.  A SIMD so holds two waves, and one issues
@@ -219,6 +247,7 @@ __device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
 template <typename T, bool AKC, bool BKC, int EPI, int FM, int FN>
 __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
   using G = Geo<FM, FN>;
+  constexpr int kStages = G::kStages;
   constexpr int ES = sizeof(typename T::storage);  // 2 or 4
   constexpr int BK = kRowBytes / ES;               // 64 or 32 k values per K tile
   constexpr bool F32IN = ES == 4;
@@ -361,10 +390,17 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
   };
   constexpr int kLoads = FM + FN;  // direct loads per thread and K tile
   // Waits until at most `newer` whole tiles of this thread's direct loads are pending.
+  static_assert((kStages - 2) * kLoads < 64, "vmcnt is a 6-bit counter");
   auto wait_tiles = [&](int newer) {
-    if (newer >= 2) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * kLoads) : "memory");
-    else if (newer == 1) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kLoads) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    switch (newer) {
+      case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+      case 1: asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kLoads) : "memory"); break;
+      case 2: asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * kLoads) : "memory"); break;
+      case 3: asm volatile("s_waitcnt vmcnt(%0)" : : "n"(3 * kLoads) : "memory"); break;
+      case 4: asm volatile("s_waitcnt vmcnt(%0)" : : "n"(4 * kLoads) : "memory"); break;
+      case 5: asm volatile("s_waitcnt vmcnt(%0)" : : "n"(5 * kLoads) : "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(%0)" : : "n"(6 * kLoads) : "memory"); break;
+    }
   };
 
   // ---- fragment reads.  This wave takes sub-steps ks0, ks0 + 1 of every K
@@ -481,18 +517,20 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
   const std::integral_constant<int, 0> J0;
   const std::integral_constant<int, 1> J1;
 
-  // One K tile.  MORE: another tile follows; T2, T3: tiles kt + 2, kt + 3 exist;
-  // LAST: tile kt + 3 is the last one and may be partly filled.
-  auto k_tile = [&](int kt, auto MORE, auto T2, auto T3, auto LAST) {
-    constexpr bool more = decltype(MORE)::value, t2 = decltype(T2)::value, t3 = decltype(T3)::value;
+  // One K tile.  MORE: another tile follows; PEND: how many of the tiles kt + 2 .. kt + kStages - 2 exist
+  // (their loads may stay pending); ISSUE: tile kt + kStages - 1 exists and is asked for now;
+  // LAST: it is the last one and may be partly filled.
+  auto k_tile = [&](int kt, auto MORE, auto PEND, auto ISSUE, auto LAST) {
+    constexpr bool more = decltype(MORE)::value, t3 = decltype(ISSUE)::value;
+    constexpr int pend = decltype(PEND)::value;
     constexpr bool last = decltype(LAST)::value;
     __builtin_amdgcn_sched_barrier(0);
     if (more) {
       // Tile kt + 1 is needed from here on (the refills below read it): its
-      // loads have landed once only those of tile kt + 2 are pending.  After
+      // loads have landed once only those of the tiles behind it are pending.  After
       // the barrier every wave's share is in LDS and every wave has finished
-      // reading tile kt - 1, whose stage the loads of tile kt + 3 overwrite.
-      wait_tiles(t2 ? 1 : 0);
+      // reading tile kt - 1, whose stage the loads of tile kt + kStages - 1 overwrite.
+      wait_tiles(pend);
       __builtin_amdgcn_s_barrier();
       if (t3) {
         if (last && k_rem != 0) issue_last_tile((kt + kStages - 1) % kStages);
@@ -519,7 +557,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
     if (more) issue_frags(J1);
   };
 
-  // Tiles 0 .. 2 go out at once; tile kt + 3 follows at the barrier of K tile kt.
+  // Tiles 0 .. kStages - 2 go out at once; tile kt + kStages - 1 follows at the barrier of K tile kt.
 #pragma unroll
   for (int s = 0; s < kStages - 1; ++s)
     if (s < KT) {
@@ -535,11 +573,15 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
     const std::true_type yes;
     const std::false_type no;
     int kt = 0;
-    for (; kt + 4 < KT; ++kt) k_tile(kt, yes, yes, yes, no);
-    if (kt + 3 < KT) k_tile(kt++, yes, yes, yes, yes);
-    if (kt + 2 < KT) k_tile(kt++, yes, yes, no, no);
-    if (kt + 1 < KT) k_tile(kt++, yes, no, no, no);
-    k_tile(kt, no, no, no, no);
+    // Steady state: every tile up to kt + kStages exists.  Then the tile that asks for the last one, the
+    // tiles that ask for nothing (one pending tile fewer each), and the last tile.
+    for (; kt + kStages < KT; ++kt) k_tile(kt, yes, std::integral_constant<int, kStages - 3>{}, yes, no);
+    if (kt + kStages - 1 < KT) k_tile(kt++, yes, std::integral_constant<int, kStages - 3>{}, yes, yes);
+    tail_tiles<kStages - 2>([&](auto R) {  // R tiles follow this one
+      constexpr int r = decltype(R)::value;
+      if (kt + r < KT) k_tile(kt++, yes, std::integral_constant<int, r - 1>{}, no, no);
+    });
+    k_tile(kt, no, std::integral_constant<int, 0>{}, no, no);
   }
 
   {
@@ -744,7 +786,7 @@ int launch_epi(ginn_hip_ctx* ctx, const MidParams& p, int batch, int splits, int
   const dim3 grid(p.tiles_m * p.tiles_n, batch, splits);
   // Only the stages a short K loop touches are allocated (at least two: the
   // epilogue staging lives there), so that more workgroups fit on a CU then.
-  const int stages = p.k_tiles < 2 ? 2 : (p.k_tiles < kStages ? p.k_tiles : kStages);
+  const int stages = p.k_tiles < 2 ? 2 : (p.k_tiles < G::kStages ? p.k_tiles : G::kStages);
   const int lds_bytes = stages * G::kStageBytes;
 #define GH_MID_LAUNCH(E)                                                                          \
   {                                                                                               \
