@@ -434,6 +434,12 @@ int launch_gemm_ksplit(ginn_hip_ctx* ctx, const GemmArgs& args);
 enum IntOp { kIntAdd = 0, kIntSub, kIntMul, kIntMax, kIntScaleShift, kIntMulAdd };
 int launch_int_arith(ginn_hip_ctx* ctx, int op, size_t n, size_t rows, const void* a, const void* b, const void* c,
                      int ia, int ib, void* dst, int accumulate);
+// Select, Mask (forward, no accumulation) and UpperTri on 32-bit integers; operands checked by the callers.
+int launch_int_select(ginn_hip_ctx* ctx, size_t n, const unsigned char* cond, const void* a, int a_is_scalar,
+                      const void* b, int b_is_scalar, void* dst);
+int launch_int_mask(ginn_hip_ctx* ctx, size_t mask_size, size_t n, const void* mask, int value, const void* x,
+                    void* dst);
+int launch_int_upper_tri(ginn_hip_ctx* ctx, size_t n, void* dst);
 // Bandwidth-oriented kernel for narrow right-hand sides (n <= 64).
 int launch_gemm_skinny(ginn_hip_ctx* ctx, const GemmArgs& args);
 int launch_gemm_strip(ginn_hip_ctx* ctx, const GemmArgs& args);

@@ -412,6 +412,10 @@ using namespace ginn_hip;
 #define GH_ENTER(name, ctx)                                                    \
   GH_CHECK_ARG(ctx, name ": ctx is NULL");                                     \
   GH_CHECK_ARG(dtype_valid(dtype), name ": unknown dtype %d", dtype)
+// The same for entry points that also take 32-bit integers.
+#define GH_ENTER_OR_INT(name, ctx)                                             \
+  GH_CHECK_ARG(ctx, name ": ctx is NULL");                                     \
+  GH_CHECK_ARG(dtype_valid(dtype) || dtype == GINN_HIP_I32, name ": unknown dtype %d", dtype)
 
 extern "C" {
 
@@ -487,9 +491,10 @@ int ginn_hip_dropout_mask(ginn_hip_ctx* ctx, size_t n, float p, unsigned long lo
 
 int ginn_hip_select(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n, const unsigned char* cond, const void* a,
                     int a_is_scalar, const void* b, int b_is_scalar, void* dst) {
-  GH_ENTER("ginn_hip_select", ctx);
+  GH_ENTER_OR_INT("ginn_hip_select", ctx);
   if (n == 0) return kOk;
   GH_CHECK_ARG(cond && a && b && dst, "ginn_hip_select: NULL operand");
+  if (dtype == GINN_HIP_I32) return launch_int_select(ctx, n, cond, a, a_is_scalar, b, b_is_scalar, dst);
   GH_HIP(hipSetDevice(ctx->device));
   const unsigned grid = grid_for(n, kBlock, ctx->num_cus);
   GH_DISPATCH_DTYPE(dtype, (select_kernel<T><<<grid, kBlock, 0, ctx->stream>>>(
@@ -519,10 +524,14 @@ int ginn_hip_select_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n, const
 
 int ginn_hip_mask_select(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t mask_size, size_t batch, const void* mask,
                          float value, const void* x, void* dst, int accumulate) {
-  GH_ENTER("ginn_hip_mask_select", ctx);
+  GH_ENTER_OR_INT("ginn_hip_mask_select", ctx);
   const size_t n = mask_size * batch;
   if (n == 0) return kOk;
   GH_CHECK_ARG(mask && x && dst, "ginn_hip_mask_select: NULL operand");
+  if (dtype == GINN_HIP_I32) {
+    GH_CHECK_ARG(!accumulate, "ginn_hip_mask_select: 32-bit integers have no gradient to accumulate");
+    return launch_int_mask(ctx, mask_size, n, mask, static_cast<int>(value), x, dst);
+  }
   GH_HIP(hipSetDevice(ctx->device));
   const unsigned grid = grid_for(n, kBlock, ctx->num_cus);
   GH_DISPATCH_DTYPE(dtype, (mask_select_kernel<T><<<grid, kBlock, 0, ctx->stream>>>(

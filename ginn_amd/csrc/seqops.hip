@@ -798,6 +798,7 @@ int ginn_hip_upper_tri(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int n, void* dst
   GH_CHECK_ARG(n >= 0, "ginn_hip_upper_tri: negative size");
   if (n == 0) return kOk;
   GH_CHECK_ARG(dst, "ginn_hip_upper_tri: NULL pointer");
+  if (dtype == GINN_HIP_I32) return launch_int_upper_tri(ctx, static_cast<size_t>(n), dst);
   GH_HIP(hipSetDevice(ctx->device));
   const unsigned grid = grid_for(static_cast<size_t>(n) * n, kBlock, ctx->num_cus);
   GH_DISPATCH_DTYPE(dtype, (upper_tri_kernel<T><<<grid, kBlock, 0, ctx->stream>>>(n, static_cast<T::storage*>(dst))));

@@ -292,15 +292,16 @@ class ColBroadcastNode : public BaseDataNode<Scalar> {
     if (cols > 1) {
       internal::require_gpu(this->dev(), "ColBroadcast");
       value().resize(x.rows(), cols);
-      GINN_HIP_CALL(ginn_hip_col_broadcast(internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(x.rows()),
+      GINN_HIP_CALL(ginn_hip_col_broadcast(internal::ctx_of(x), internal::move_dtype_of<Scalar>(), static_cast<int>(x.rows()),
                                            static_cast<int>(cols), x.data(), value().data()));
     } else {
       value().map(in_->value(), in_->value().shape());
     }
   }
   void backward_() override {
-    if (in_->has_grad() && cols_->value() > 1)
-      GINN_HIP_CALL(ginn_hip_row_sum(internal::ctx_of(grad()), dtype_of<Scalar>(), static_cast<int>(grad().rows()),
+    if constexpr (is_floating_point_v<Scalar>)
+      if (in_->has_grad() && cols_->value() > 1)
+        GINN_HIP_CALL(ginn_hip_row_sum(internal::ctx_of(grad()), dtype_of<Scalar>(), static_cast<int>(grad().rows()),
                                      static_cast<int>(grad().cols()), grad().data(), in_->grad().data(), 1));
   }
 
@@ -561,8 +562,10 @@ class PermuteNode : public BaseDataNode<Scalar>, public internal::SliceProvider<
     internal::require_gpu(dst.dev(), "Permute");
     std::vector<long long> dims(src_shape.begin(), src_shape.end());
     std::vector<int> p(perm.begin(), perm.end());
-    GINN_HIP_CALL(ginn_hip_permute(internal::ctx_of(dst), dtype_of<Scalar>(), static_cast<int>(dims.size()),
-                                   dims.data(), p.data(), src.data(), dst.data(), accumulate ? 1 : 0));
+    if constexpr (!is_floating_point_v<Scalar>) GINN_ASSERT(!accumulate, "integers are moved, not summed");
+    GINN_HIP_CALL(ginn_hip_permute(internal::ctx_of(dst), internal::move_dtype_of<Scalar>(),
+                                   static_cast<int>(dims.size()), dims.data(), p.data(), src.data(), dst.data(),
+                                   accumulate ? 1 : 0));
   }
   Tensor<Scalar>& raw_value() const { return const_cast<Tensor<Scalar>&>(BaseDataNode<Scalar>::value()); }
   internal::SliceTaker<Scalar>* pending_product() const {
@@ -608,7 +611,7 @@ class PermuteNode : public BaseDataNode<Scalar>, public internal::SliceProvider<
       skip_backward_ = false;
       return;
     }
-    if (!in_->has_grad()) return;
+    if (!in_->has_grad() || !is_floating_point_v<Scalar>) return;  // (integers carry no gradient)
     if (overwrite_) {
       // grad() is in's gradient storage under the permuted shape: permute into a
       // temporary and copy back (the reference's `.eval()`, ginn/node/layout.h:766-770).
@@ -813,12 +816,13 @@ class RowBroadcastNode : public BaseDataNode<Scalar> {
     GINN_ASSERT(x.rows() == 1);
     const Size rows = rows_->value();
     value().resize(rows, x.cols());
-    GINN_HIP_CALL(ginn_hip_row_broadcast(internal::ctx_of(x), dtype_of<Scalar>(), static_cast<int>(rows),
+    GINN_HIP_CALL(ginn_hip_row_broadcast(internal::ctx_of(x), internal::move_dtype_of<Scalar>(), static_cast<int>(rows),
                                          static_cast<int>(x.cols()), x.data(), value().data()));
   }
   void backward_() override {
-    if (in_->has_grad())
-      GINN_HIP_CALL(ginn_hip_col_sum(internal::ctx_of(grad()), dtype_of<Scalar>(), static_cast<int>(grad().rows()),
+    if constexpr (is_floating_point_v<Scalar>)
+      if (in_->has_grad())
+        GINN_HIP_CALL(ginn_hip_col_sum(internal::ctx_of(grad()), dtype_of<Scalar>(), static_cast<int>(grad().rows()),
                                      static_cast<int>(grad().cols()), grad().data(), in_->grad().data(), 1));
   }
 
@@ -847,7 +851,7 @@ class UpperTriNode : public BaseDataNode<Scalar> {
       return;
     }
     internal::require_gpu(this->dev(), "UpperTri");
-    GINN_HIP_CALL(ginn_hip_upper_tri(internal::ctx_of(value()), dtype_of<Scalar>(), static_cast<int>(s),
+    GINN_HIP_CALL(ginn_hip_upper_tri(internal::ctx_of(value()), arith_dtype_of<Scalar>(), static_cast<int>(s),
                                      value().data()));
   }
 

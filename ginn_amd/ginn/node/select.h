@@ -11,10 +11,10 @@ namespace ginn {
 
 // value[i] = if[i] ? then[i] : else[i]; a branch of shape {} is one value used
 // everywhere, and its gradient is the sum over the selected entries
-// (ginn/node/select.h:24-112).
+// (ginn/node/select.h:24-112).  On Int the forward pass alone (integers carry
+// no gradient here).
 template <typename Scalar>
 class SelectNode : public BaseDataNode<Scalar> {
-  static_assert(is_floating_point_v<Scalar>, "Select computes on Real, Half and BFloat16 tensors in this build");
   NodePtr<bool> if_;
   NodePtr<Scalar> then_, else_;
 
@@ -26,18 +26,20 @@ class SelectNode : public BaseDataNode<Scalar> {
     GINN_ASSERT(is_scalar(then_) || then_->shape() == if_->shape());
     GINN_ASSERT(is_scalar(else_) || else_->shape() == if_->shape());
     value().resize(if_->shape());
-    GINN_HIP_CALL(ginn_hip_select(internal::ctx_of(value()), dtype_of<Scalar>(), static_cast<size_t>(value().size()),
+    GINN_HIP_CALL(ginn_hip_select(internal::ctx_of(value()), arith_dtype_of<Scalar>(), static_cast<size_t>(value().size()),
                                   cond(), then_->value().data(), is_scalar(then_) ? 1 : 0, else_->value().data(),
                                   is_scalar(else_) ? 1 : 0, value().data()));
   }
   void backward_() override {
-    const size_t n = static_cast<size_t>(grad().size());
-    if (then_->has_grad())
-      GINN_HIP_CALL(ginn_hip_select_bwd(internal::ctx_of(grad()), dtype_of<Scalar>(), n, cond(), 1, grad().data(),
-                                        then_->grad().data(), is_scalar(then_) ? 1 : 0));
-    if (else_->has_grad())
-      GINN_HIP_CALL(ginn_hip_select_bwd(internal::ctx_of(grad()), dtype_of<Scalar>(), n, cond(), 0, grad().data(),
-                                        else_->grad().data(), is_scalar(else_) ? 1 : 0));
+    if constexpr (is_floating_point_v<Scalar>) {
+      const size_t n = static_cast<size_t>(grad().size());
+      if (then_->has_grad())
+        GINN_HIP_CALL(ginn_hip_select_bwd(internal::ctx_of(grad()), dtype_of<Scalar>(), n, cond(), 1, grad().data(),
+                                          then_->grad().data(), is_scalar(then_) ? 1 : 0));
+      if (else_->has_grad())
+        GINN_HIP_CALL(ginn_hip_select_bwd(internal::ctx_of(grad()), dtype_of<Scalar>(), n, cond(), 0, grad().data(),
+                                          else_->grad().data(), is_scalar(else_) ? 1 : 0));
+    }
   }
 
  public:
@@ -90,7 +92,7 @@ class MaskNode : public BaseDataNode<Scalar> {
 
   void run(const Tensor<Scalar>& x, float val, Tensor<Scalar>& dst, bool accumulate) {
     const Size ms = mask_->value().size();
-    GINN_HIP_CALL(ginn_hip_mask_select(internal::ctx_of(dst), dtype_of<Scalar>(), static_cast<size_t>(ms),
+    GINN_HIP_CALL(ginn_hip_mask_select(internal::ctx_of(dst), arith_dtype_of<Scalar>(), static_cast<size_t>(ms),
                                        static_cast<size_t>(x.size() / ms), mask_->value().data(), val, x.data(),
                                        dst.data(), accumulate ? 1 : 0));
   }
@@ -106,7 +108,8 @@ class MaskNode : public BaseDataNode<Scalar> {
     run(in_->value(), mask_val_, value(), false);
   }
   void backward_() override {
-    if (in_->has_grad()) run(grad(), 0.f, in_->grad(), true);
+    if constexpr (is_floating_point_v<Scalar>)
+      if (in_->has_grad()) run(grad(), 0.f, in_->grad(), true);
   }
 
  public:

@@ -212,7 +212,7 @@ void bind_node_types(py::module_& m) {
 }
 
 // The nodes that exist for Int as well as for the floating scalars (ginn-py/node/common-py.cu.cpp:34-70,
-// ginn-py/node/layout-py.cu.cpp): arithmetic, layout, comparison.
+// ginn-py/node/layout-py.cu.cpp, ginn-py/node/select-py.cu.cpp:33-46): arithmetic, layout, comparison, selection.
 template <typename S>
 void bind_shared_nodes(py::module_& m) {
   using N = Node<S>;
@@ -241,6 +241,18 @@ void bind_shared_nodes(py::module_& m) {
     return as_node(Stack<S>(g));
   });
   m.def("LessThan", [P](In a, In b) { return SP<Node<bool>>(LessThan(P(a), P(b)).as_shared_ptr()); });
+  m.def("Permute", [P](In x, const Shape& s) { return as_node(Permute(P(x), s)); });
+  m.def("Transpose", [P](In x, Size i, Size j) { return as_node(Transpose(P(x), i, j)); });
+  m.def("RowBroadcast", [P](In x, Size rows) { return as_node(RowBroadcast(P(x), rows)); });
+  m.def("ColBroadcast", [P](In x, Size cols) { return as_node(ColBroadcast(P(x), cols)); });
+  m.def("Mask", [P](In x, In mask, double val) { return as_node(Mask(P(x), P(mask), val)); });
+  m.def("Select", [P](const SP<Node<bool>>& c, In a, In b) { return as_node(Select(NodePtr<bool>(c), P(a), P(b))); });
+  m.def("Select", [P](const SP<Node<bool>>& c, In a, double b) {
+    return as_node(Select(NodePtr<bool>(c), P(a), S(static_cast<float>(b))));
+  });
+  m.def("Select", [P](const SP<Node<bool>>& c, double a, In b) {
+    return as_node(Select(NodePtr<bool>(c), S(static_cast<float>(a)), P(b)));
+  });
 }
 
 // Everything that computes, for one floating scalar type: overloads of the
@@ -276,12 +288,6 @@ void bind_float_nodes(py::module_& m) {
   GINN_PY_UNARY(LayerNorm);
 #undef GINN_PY_UNARY
   m.def("AxisSum", [P](In x, const std::vector<Size>& axes) { return as_node(AxisSum(P(x), axes)); });
-  m.def("Permute", [P](In x, const Shape& s) { return as_node(Permute(P(x), s)); });
-  m.def("Transpose", [P](In x, Size i, Size j) { return as_node(Transpose(P(x), i, j)); });
-  m.def("RowBroadcast", [P](In x, Size rows) { return as_node(RowBroadcast(P(x), rows)); });
-  m.def("ColBroadcast", [P](In x, Size cols) { return as_node(ColBroadcast(P(x), cols)); });
-  m.def("Mask", [P](In x, In mask, double val) { return as_node(Mask(P(x), P(mask), val)); });
-  m.def("Select", [P](const SP<Node<bool>>& c, In a, In b) { return as_node(Select(NodePtr<bool>(c), P(a), P(b))); });
   auto index_of = [](const SP<DataNode<Int>>& i) { return DataPtr<Int>(i); };
   m.def("Pick", [P, index_of](In x, const SP<DataNode<Int>>& i) { return as_node(Pick(P(x), index_of(i))); });
   m.def("Pick", [P](In x, const std::vector<Int>& i) { return as_node(Pick(P(x), i)); });
@@ -438,6 +444,12 @@ PYBIND11_MODULE(ginn, m) {
         auto out = cast_data<Int>(n);
         out->set_has_grad(false);
         return out;
+      })
+      // conditions of Select (ginn-py/test/test_nodes.py:679)
+      .def("bool", [](DataNode<Real>& n) {
+        auto out = cast_data<bool>(n);
+        out->set_has_grad(false);
+        return out;
       });
 
   m.def("Data", [](const py::array& a) {
@@ -447,6 +459,18 @@ PYBIND11_MODULE(ginn, m) {
     return SP<DataNode<Real>>(n.as_shared_ptr());
   });
   m.def("Data", &data_node, py::arg("dev"), py::arg("shape"), py::arg("scalar") = Scalar_::Real);
+  // UpperTri(dev, size, scalar) (ginn-py/node/layout-py.cu.cpp:30-46,113-125)
+  m.def("UpperTri",
+        [](const DevPtr& dev, Size size, Scalar_ s) -> py::object {
+          switch (s) {
+            case Scalar_::Real: return py::cast(as_node(UpperTri<Real>(dev, size)));
+            case Scalar_::Half: return py::cast(as_node(UpperTri<Half>(dev, size)));
+            case Scalar_::BFloat16: return py::cast(as_node(UpperTri<BFloat16>(dev, size)));
+            case Scalar_::Int: return py::cast(as_node(UpperTri<Int>(dev, size)));
+            default: GINN_THROW("UpperTri exists for Real, Half, BFloat16 and Int");
+          }
+        },
+        py::arg("dev"), py::arg("size"), py::arg("scalar") = Scalar_::Real);
   // Values(dev, nested list): a Real data node holding the literal (ginn/node/data.h:211-221)
   m.def("Values", [](const DevPtr& dev, const py::object& nested) {
     auto arr = py::array_t<Real, py::array::f_style | py::array::forcecast>::ensure(nested);

@@ -581,7 +581,7 @@ int ginn_hip_scaled_masked_softmax_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
                                        void* dx);
 
 /* UpperTriNode (ginn/node/layout.h:922-955): dst [n x n] = 1 where
- * row <= col, else 0. */
+ * row <= col, else 0.  dtype may be GINN_HIP_I32. */
 int ginn_hip_upper_tri(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, int n,
                        void* dst);
 
@@ -633,7 +633,8 @@ int ginn_hip_mask_scale(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
 /* SelectNode (ginn/node/select.h:24-112): dst[i] = cond[i] ? a : b, cond one
  * byte per element (Tensor<bool>); a branch flagged scalar is a single value
  * used for every i.  Backward: dst[i] += dy[i] where (cond[i] != 0) == want,
- * summed into dst[0] when the branch is a single value. */
+ * summed into dst[0] when the branch is a single value.  ginn_hip_select also
+ * takes GINN_HIP_I32 (Select on Int, test/nodes.cu.cpp:825). */
 int ginn_hip_select(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
                     const unsigned char* cond, const void* a, int a_is_scalar,
                     const void* b, int b_is_scalar, void* dst);
@@ -643,7 +644,9 @@ int ginn_hip_select_bwd(ginn_hip_ctx* ctx, ginn_hip_dtype dtype, size_t n,
 
 /* MaskNode (ginn/node/select.h:114-187): x viewed as [mask_size x batch];
  * dst (+)= mask != 0 ? x : value.  Forward with `value` = the mask value,
- * backward on the gradient with value 0 and accumulate. */
+ * backward on the gradient with value 0 and accumulate.  dtype may be
+ * GINN_HIP_I32 without accumulate (Mask on Int, test/nodes.cu.cpp:860): value
+ * is then truncated to an integer. */
 int ginn_hip_mask_select(ginn_hip_ctx* ctx, ginn_hip_dtype dtype,
                          size_t mask_size, size_t batch, const void* mask,
                          float value, const void* x, void* dst, int accumulate);

@@ -492,6 +492,107 @@ void arithmetic_goldens() {
   EXPECT_VALUES(CwiseMax(N(b), N(c)), s, {1, 2, 3, 4, 5, 6});
 }
 
+// Select, Mask, Permute / Transpose / InPlacePermute, RowBroadcast / ColBroadcast and UpperTri with the known
+// answers of test/nodes.cu.cpp:326-441, 825-880, forward, for the floating scalars and for Int (fractions are
+// truncated by the cast to Int exactly as the reference's cast<Int>() truncates them).
+template <typename Scalar>
+void select_goldens() {
+  using N = NodePtr<Scalar>;
+  constexpr bool is_int = std::is_same_v<Scalar, Int>;
+  // what a value turns into when it is stored as Scalar and read back
+  auto q = [](float v) { return static_cast<float>(Scalar(v)); };
+  auto qs = [&](std::vector<float> v) {
+    for (auto& x : v) x = q(x);
+    return v;
+  };
+  {  // Select (:825-858)
+    auto if_ = Values<2>({{1., 0.}, {0., 1.}, {1., 0.}})->template cast<bool>();
+    if_->move_to(gpu());
+    if_->set_has_grad(false);
+    auto a = on_gpu<Scalar>(Values<2>({{1., 2.}, {3., 4.}, {5., 6.}}));
+    auto b = on_gpu<Scalar>(Values<2>({{.1, .2}, {.3, .4}, {.5, .6}}));
+    const Shape s{3, 2};
+    expect_values<Scalar>(__LINE__, Select(if_, N(a), N(b)), s, qs({1, .3f, 5, .2f, 4, .6f}));
+    expect_values<Scalar>(__LINE__, Select(if_, N(a), Scalar(7)), s, {1, 7, 5, 7, 4, 7});
+    expect_values<Scalar>(__LINE__, Select(if_, Scalar(7), N(b)), s, qs({7, .3f, 7, .2f, 7, .6f}));
+    expect_values<Scalar>(__LINE__, Select(if_, Scalar(7), Scalar(-2)), s, {7, -2, 7, -2, 7, -2});
+    if (is_int) CHECK(q(.3f) == 0.f);
+  }
+  {  // Mask (:860-885): a full mask and one that broadcasts over the columns
+    auto mask = on_gpu<Scalar>(Values<2>({{1., 0.}, {0., 1.}, {1., 0.}}));
+    auto mask2 = on_gpu<Scalar>(Values<2>({{1.}, {0.}, {1.}}));
+    auto a = on_gpu<Scalar>(Values<2>({{1., 2.}, {3., 4.}, {5., 6.}}));
+    EXPECT_VALUES(Mask(N(a), N(mask), Scalar(-1)), (Shape{3, 2}), {1, -1, 5, -1, 4, -1});
+    EXPECT_VALUES(Mask(N(a), N(mask2), Scalar(7)), (Shape{3, 2}), {1, 7, 5, 2, 7, 6});
+  }
+  {  // Permute / Transpose / InPlacePermute (:326-380): a[i][j][k] = 1 + k + 4 j + 8 i, shape {3, 2, 4}
+    const Shape dims{3, 2, 4};
+    std::vector<float> av(24);
+    for (int k = 0; k < 4; ++k)
+      for (int j = 0; j < 2; ++j)
+        for (int i = 0; i < 3; ++i) av[i + 3 * (j + 2 * k)] = 1.f + k + 4 * j + 8 * i;
+    auto a0 = Values<3>({{{1, 2, 3, 4}, {5, 6, 7, 8}},
+                         {{9, 10, 11, 12}, {13, 14, 15, 16}},
+                         {{17, 18, 19, 20}, {21, 22, 23, 24}}});
+    auto a = on_gpu<Scalar>(a0);
+    expect_values<Scalar>(__LINE__, N(a) * 1, dims, av);  // the literal is laid out as the formula says
+    // result[x] = a[y] with x[n] = y[perm[n]]
+    auto permuted = [&](const Shape& perm, Shape& out_dims) {
+      out_dims = {dims[perm[0]], dims[perm[1]], dims[perm[2]]};
+      std::vector<float> w(24);
+      Size y[3];
+      for (y[2] = 0; y[2] < dims[2]; ++y[2])
+        for (y[1] = 0; y[1] < dims[1]; ++y[1])
+          for (y[0] = 0; y[0] < dims[0]; ++y[0]) {
+            const Size x0 = y[perm[0]], x1 = y[perm[1]], x2 = y[perm[2]];
+            w[x0 + out_dims[0] * (x1 + out_dims[1] * x2)] = av[y[0] + 3 * (y[1] + 2 * y[2])];
+          }
+      return w;
+    };
+    Shape od;
+    {  // entries of the reference's literals b (perm 0 2 1), c (2 1 0) and e (1 2 0)
+      auto w = permuted(Shape{0, 2, 1}, od);
+      CHECK((od == Shape{3, 4, 2}));
+      CHECK(w[0 + 3 * (1 + 4 * 0)] == 2.f && w[1 + 3 * (0 + 4 * 1)] == 13.f && w[2 + 3 * (3 + 4 * 1)] == 24.f);
+      w = permuted(Shape{2, 1, 0}, od);
+      CHECK((od == Shape{4, 2, 3}));
+      CHECK(w[0 + 4 * (0 + 2 * 1)] == 9.f && w[1 + 4 * (1 + 2 * 2)] == 22.f && w[3 + 4 * (0 + 2 * 1)] == 12.f);
+      w = permuted(Shape{1, 2, 0}, od);
+      CHECK((od == Shape{2, 4, 3}));
+      CHECK(w[0 + 2 * (1 + 4 * 1)] == 10.f && w[1 + 2 * (3 + 4 * 2)] == 24.f && w[1 + 2 * (0 + 4 * 1)] == 13.f);
+    }
+    for (const Shape& perm : {Shape{0, 2, 1}, Shape{2, 1, 0}, Shape{1, 0, 2}, Shape{1, 2, 0}, Shape{2, 0, 1},
+                              Shape{0, 1, 2}}) {
+      const auto w = permuted(perm, od);
+      expect_values<Scalar>(__LINE__, Permute(N(a), perm), od, w);
+      expect_values<Scalar>(__LINE__, InPlacePermute(N(a) * 1, perm), od, w);
+    }
+    expect_values<Scalar>(__LINE__, Transpose(N(a), 1, 2), Shape{3, 4, 2}, permuted(Shape{0, 2, 1}, od));
+    expect_values<Scalar>(__LINE__, Transpose(N(a), 2, 0), Shape{4, 2, 3}, permuted(Shape{2, 1, 0}, od));
+    expect_values<Scalar>(__LINE__, Transpose(N(a), 0, 1), Shape{2, 3, 4}, permuted(Shape{1, 0, 2}, od));
+  }
+  {  // RowBroadcast / ColBroadcast (:382-421)
+    auto a = on_gpu<Scalar>(Values<2>({{1}, {2}, {3}}));
+    auto b = on_gpu<Scalar>(Values<2>({{0.1, 1.2, 2.3}}));
+    const auto b3 = qs({.1f, .1f, .1f, 1.2f, 1.2f, 1.2f, 2.3f, 2.3f, 2.3f});
+    expect_values<Scalar>(__LINE__, RowBroadcast(N(b), 3), Shape{3, 3}, b3);
+    expect_values<Scalar>(__LINE__, RowBroadcast(N(b), 1), Shape{1, 3}, qs({.1f, 1.2f, 2.3f}));
+    expect_values<Scalar>(__LINE__, RowBroadcast(N(b), Dim(a, 0)), Shape{3, 3}, b3);
+    expect_values<Scalar>(__LINE__, RowBroadcast(N(b), Dim(a, 1)), Shape{1, 3}, qs({.1f, 1.2f, 2.3f}));
+    EXPECT_VALUES(ColBroadcast(N(a), 3), (Shape{3, 3}), {1, 2, 3, 1, 2, 3, 1, 2, 3});
+    EXPECT_VALUES(ColBroadcast(N(a), 1), (Shape{3, 1}), {1, 2, 3});
+    EXPECT_VALUES(ColBroadcast(N(a), Dim(b, 1)), (Shape{3, 3}), {1, 2, 3, 1, 2, 3, 1, 2, 3});
+    EXPECT_VALUES(ColBroadcast(N(a), Dim(b, 0)), (Shape{3, 1}), {1, 2, 3});
+  }
+  {  // UpperTri (:423-441)
+    EXPECT_VALUES(UpperTri<Scalar>(gpu(), 2), (Shape{2, 2}), {1, 0, 1, 1});
+    std::vector<float> tri5(25);
+    for (int c = 0; c < 5; ++c)
+      for (int r = 0; r < 5; ++r) tri5[r + 5 * c] = r <= c ? 1.f : 0.f;
+    expect_values<Scalar>(__LINE__, UpperTri<Scalar>(gpu(), 5), Shape{5, 5}, tri5);
+  }
+}
+
 extern "C" {
 
 // Runs the named group of checks; returns the report of failed checks ("" = all passed).
@@ -534,6 +635,11 @@ const char* shim_structural(const char* which) {
       arithmetic_goldens<Half>();
       arithmetic_goldens<BFloat16>();
       arithmetic_goldens<Int>();
+    } else if (w == "select_goldens") {
+      select_goldens<Real>();
+      select_goldens<Half>();
+      select_goldens<BFloat16>();
+      select_goldens<Int>();
     } else if (w == "arena_limits") {
       arena_limits();
     } else {

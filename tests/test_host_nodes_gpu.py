@@ -198,7 +198,7 @@ def test_nonlin_nodes(shim, dt, act):
 
 @pytest.mark.parametrize("case", ["tensor_ctors", "tensor_ops", "forwardedness", "gradfulness", "arena_tensors",
                                   "arena_nodes", "arena_limits", "layout_goldens",
-                                  "arithmetic_goldens"])
+                                  "arithmetic_goldens", "select_goldens"])
 def test_reference_structural_cases(shim, case):
     """The reference's structural tests on the HIP device: Tensor construction /
     copy / move / assignment across devices, resize, set, serialize and errors

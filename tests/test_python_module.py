@@ -310,6 +310,30 @@ def test_int_nodes_through_the_bindings(ginn):
     lt = x < y
     ginn.Graph(lt).forward()
     assert lt.value.list() == [True, True, False, False, False]
+    # selection (ginn-py/test/test_nodes.py:678-730); the fractions of the reference's case truncate to 0
+    if_ = ginn.Values(dev, [[1, 0], [0, 1], [1, 0]]).bool()
+    s1 = vals([[1, 2], [3, 4], [5, 6]])
+    s2 = vals([[0.1, 0.2], [0.3, 0.4], [0.5, 0.6]])
+    check(ginn.Select(if_, s1, s2), [[1, 0], [0, 4], [5, 0]])
+    check(ginn.Select(if_, s1, 7), [[1, 7], [7, 4], [5, 7]])
+    check(ginn.Select(if_, 7, s2), [[7, 0], [0, 7], [7, 0]])
+    mask, mask2 = vals([[1, 0], [0, 1], [1, 0]]), vals([[1], [0], [1]])
+    check(ginn.Mask(s1, mask, -1), [[1, -1], [-1, 4], [5, -1]])
+    check(ginn.Mask(s1, mask2, 7), [[1, 2], [7, 7], [5, 6]])
+    # axis orders (:245-300), broadcasts (:303-366), UpperTri (:369-385)
+    t = vals([[[1, 2, 3, 4], [5, 6, 7, 8]], [[9, 10, 11, 12], [13, 14, 15, 16]],
+              [[17, 18, 19, 20], [21, 22, 23, 24]]])
+    tn = np.arange(1, 25).reshape(3, 2, 4)
+    for perm in ([0, 2, 1], [2, 1, 0], [1, 0, 2], [1, 2, 0], [2, 0, 1], [0, 1, 2]):
+        check(ginn.Permute(t, perm), tn.transpose(perm).tolist())
+    check(ginn.Transpose(t, 2, 0), tn.transpose(2, 1, 0).tolist())
+    col, row = vals([[1], [2], [3]]), vals([[0.1, 1.2, 2.3]])
+    check(ginn.RowBroadcast(row, 3), [[0, 1, 2]] * 3)
+    check(ginn.RowBroadcast(row, 1), [[0, 1, 2]])
+    check(ginn.ColBroadcast(col, 3), [[1, 1, 1], [2, 2, 2], [3, 3, 3]])
+    check(ginn.ColBroadcast(col, 1), [[1], [2], [3]])
+    check(ginn.UpperTri(dev, 2, I), [[1, 1], [0, 1]])
+    check(ginn.UpperTri(dev, 5, I), np.triu(np.ones((5, 5))).tolist())
 
 
 @pytest.mark.gpu
