@@ -43,8 +43,173 @@ inline const float* as_f32(const S* src, size_t ld, size_t cols, std::vector<flo
 }
 
 // C[m x n] = op(A)[m x k] * op(B)[k x n] + beta * C, column-major, fp32 accumulation, one rounding to S.
-// Blocked over K (the panel of A a column block of C reuses stays in cache) with four columns of C per sweep
-// over a column of A; a transposed A turns the sweep into dot products of contiguous columns.
+// Narrow or small products: blocked over K (the panel of A that a column block of C reuses stays in cache) with
+// four columns of C per sweep over a column of A; a transposed A turns the sweep into dot products of
+// contiguous columns.
+inline void gemm_sweep(bool ta, bool tb, int m, int n, int k, const float* a, int lda, const float* b, int ldb,
+                       float* c, int ldc) {
+  auto b_at = [&](int l, int j) { return tb ? b[j + static_cast<size_t>(l) * ldb] : b[l + static_cast<size_t>(j) * ldb]; };
+  std::vector<float> bcol(ta ? static_cast<size_t>(k) : 0);
+  for (int j0 = 0; j0 < n; j0 += 4) {
+    const int nj = std::min(4, n - j0);
+    float* cols[4];
+    for (int jj = 0; jj < 4; ++jj) cols[jj] = c + static_cast<size_t>(j0 + std::min(jj, nj - 1)) * ldc;
+    for (int jj = 0; jj < nj; ++jj) std::fill(cols[jj], cols[jj] + m, 0.f);
+    if (!ta) {
+      for (int l = 0; l < k; ++l) {
+        const float* al = a + static_cast<size_t>(l) * lda;
+        if (nj == 4) {
+          const float b0 = b_at(l, j0), b1 = b_at(l, j0 + 1), b2 = b_at(l, j0 + 2), b3 = b_at(l, j0 + 3);
+          float *c0 = cols[0], *c1 = cols[1], *c2 = cols[2], *c3 = cols[3];
+          for (int i = 0; i < m; ++i) {
+            const float v = al[i];
+            c0[i] += v * b0;
+            c1[i] += v * b1;
+            c2[i] += v * b2;
+            c3[i] += v * b3;
+          }
+        } else {
+          for (int jj = 0; jj < nj; ++jj) {
+            const float bv = b_at(l, j0 + jj);
+            float* cj = cols[jj];
+            for (int i = 0; i < m; ++i) cj[i] += al[i] * bv;
+          }
+        }
+      }
+    } else {
+      // op(A)(i, l) = A(l, i): column i of the stored A against column j of op(B)
+      for (int jj = 0; jj < nj; ++jj) {
+        for (int l = 0; l < k; ++l) bcol[static_cast<size_t>(l)] = b_at(l, j0 + jj);
+        float* cj = cols[jj];
+        for (int i = 0; i < m; ++i) {
+          const float* ai = a + static_cast<size_t>(i) * lda;
+          float sum = 0.f;
+          for (int l = 0; l < k; ++l) sum += ai[l] * bcol[static_cast<size_t>(l)];
+          cj[i] = sum;
+        }
+      }
+    }
+  }
+}
+
+// Everything else: the classic packed scheme.  op(A) is cut into blocks of kMc rows x kKc sums, stored as panels
+// of kMr rows (one sum after the other), op(B) into panels of kNr columns; a register tile of kMr x kNr sums runs
+// over one pair of panels.  Panels are padded with zeros, so the tile loop has no edges; edge tiles are stored
+// through a small buffer.  The tile loop exists twice: eight-wide with fused multiply-adds where the processor has
+// them (asked at run time: the library is built for any x86-64), and as plain loops.
+constexpr int kMr = 16, kNr = 6, kKc = 256, kMc = 128, kNc = 1536;
+
+// tile[j * kMr + i] = sum_l ap[l * kMr + i] * bp[l * kNr + j]
+inline void tile_plain(int kc, const float* ap, const float* bp, float* tile) {
+  float acc[kNr][kMr] = {};
+  for (int l = 0; l < kc; ++l, ap += kMr, bp += kNr)
+    for (int j = 0; j < kNr; ++j)
+      for (int i = 0; i < kMr; ++i) acc[j][i] += ap[i] * bp[j];
+  for (int j = 0; j < kNr; ++j)
+    for (int i = 0; i < kMr; ++i) tile[j * kMr + i] = acc[j][i];
+}
+#if defined(__x86_64__) && (defined(__GNUC__) || defined(__clang__))
+#define GINN_HOST_GEMM_HAS_FMA_TILE 1
+typedef float tile_v8 __attribute__((vector_size(32), aligned(4)));
+__attribute__((target("avx2,fma"))) inline void tile_fma(int kc, const float* ap, const float* bp, float* tile) {
+  tile_v8 acc[kNr][2] = {};
+  for (int l = 0; l < kc; ++l, ap += kMr, bp += kNr) {
+    const tile_v8 a0 = *reinterpret_cast<const tile_v8*>(ap);
+    const tile_v8 a1 = *reinterpret_cast<const tile_v8*>(ap + 8);
+#pragma GCC unroll 6
+    for (int j = 0; j < kNr; ++j) {
+      const float bj = bp[j];
+      const tile_v8 bv = {bj, bj, bj, bj, bj, bj, bj, bj};
+      acc[j][0] += a0 * bv;
+      acc[j][1] += a1 * bv;
+    }
+  }
+  for (int j = 0; j < kNr; ++j) {
+    *reinterpret_cast<tile_v8*>(tile + j * kMr) = acc[j][0];
+    *reinterpret_cast<tile_v8*>(tile + j * kMr + 8) = acc[j][1];
+  }
+}
+inline bool has_fma_tile() {
+  static const bool yes = __builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma");
+  return yes;
+}
+#else
+inline void tile_fma(int kc, const float* ap, const float* bp, float* tile) { tile_plain(kc, ap, bp, tile); }
+inline bool has_fma_tile() { return false; }
+#endif
+
+// c (fp32, leading dimension ldc) = op(a) op(b); c is overwritten.
+inline void gemm_packed(bool ta, bool tb, int m, int n, int k, const float* a, int lda, const float* b, int ldb,
+                        float* c, int ldc) {
+  const bool fma = has_fma_tile();
+  std::vector<float> apack(static_cast<size_t>(kMc) * kKc), bpack(static_cast<size_t>(kKc) * (kNc + kNr));
+  float tile[kMr * kNr];
+  for (int jc = 0; jc < n; jc += kNc) {
+    const int nc = std::min(kNc, n - jc);
+    for (int pc = 0; pc < k; pc += kKc) {
+      const int kc = std::min(kKc, k - pc);
+      // op(B)[pc .. pc + kc, jc .. jc + nc] as panels of kNr columns
+      for (int j0 = 0; j0 < nc; j0 += kNr) {
+        float* dst = bpack.data() + static_cast<size_t>(j0) * kc;
+        for (int jj = 0; jj < kNr; ++jj) {
+          const int j = jc + j0 + jj;
+          if (j0 + jj >= nc) {
+            for (int l = 0; l < kc; ++l) dst[l * kNr + jj] = 0.f;
+          } else if (tb) {  // op(B)(l, j) = B(j, l)
+            const float* src = b + j + static_cast<size_t>(pc) * ldb;
+            for (int l = 0; l < kc; ++l) dst[l * kNr + jj] = src[static_cast<size_t>(l) * ldb];
+          } else {
+            const float* src = b + pc + static_cast<size_t>(j) * ldb;
+            for (int l = 0; l < kc; ++l) dst[l * kNr + jj] = src[l];
+          }
+        }
+      }
+      for (int ic = 0; ic < m; ic += kMc) {
+        const int mc = std::min(kMc, m - ic);
+        // op(A)[ic .. ic + mc, pc .. pc + kc] as panels of kMr rows
+        for (int i0 = 0; i0 < mc; i0 += kMr) {
+          float* dst = apack.data() + static_cast<size_t>(i0) * kc;
+          const int mr = std::min(kMr, mc - i0);
+          if (ta) {  // op(A)(i, l) = A(l, i): a row of the panel is a contiguous piece of a stored column
+            for (int ii = 0; ii < kMr; ++ii) {
+              if (ii >= mr) {
+                for (int l = 0; l < kc; ++l) dst[l * kMr + ii] = 0.f;
+              } else {
+                const float* src = a + pc + static_cast<size_t>(ic + i0 + ii) * lda;
+                for (int l = 0; l < kc; ++l) dst[l * kMr + ii] = src[l];
+              }
+            }
+          } else {
+            for (int l = 0; l < kc; ++l) {
+              const float* src = a + (ic + i0) + static_cast<size_t>(pc + l) * lda;
+              for (int ii = 0; ii < mr; ++ii) dst[l * kMr + ii] = src[ii];
+              for (int ii = mr; ii < kMr; ++ii) dst[l * kMr + ii] = 0.f;
+            }
+          }
+        }
+        for (int j0 = 0; j0 < nc; j0 += kNr) {
+          const int nr = std::min(kNr, nc - j0);
+          const float* bp = bpack.data() + static_cast<size_t>(j0) * kc;
+          for (int i0 = 0; i0 < mc; i0 += kMr) {
+            const int mr = std::min(kMr, mc - i0);
+            const float* ap = apack.data() + static_cast<size_t>(i0) * kc;
+            if (fma) tile_fma(kc, ap, bp, tile);
+            else tile_plain(kc, ap, bp, tile);
+            float* out = c + (ic + i0) + static_cast<size_t>(jc + j0) * ldc;
+            if (pc == 0) {
+              for (int j = 0; j < nr; ++j)
+                for (int i = 0; i < mr; ++i) out[i + static_cast<size_t>(j) * ldc] = tile[j * kMr + i];
+            } else {
+              for (int j = 0; j < nr; ++j)
+                for (int i = 0; i < mr; ++i) out[i + static_cast<size_t>(j) * ldc] += tile[j * kMr + i];
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
 template <typename S>
 void gemm(bool ta, bool tb, int m, int n, int k, const S* A, int lda, const S* B, int ldb, float beta, S* C,
           int ldc) {
@@ -52,62 +217,26 @@ void gemm(bool ta, bool tb, int m, int n, int k, const S* A, int lda, const S* B
   std::vector<float> keep_a, keep_b;
   const float* a = as_f32(A, static_cast<size_t>(lda), static_cast<size_t>(ta ? m : k), keep_a);
   const float* b = as_f32(B, static_cast<size_t>(ldb), static_cast<size_t>(tb ? k : n), keep_b);
-  auto b_at = [&](int l, int j) { return tb ? b[j + static_cast<size_t>(l) * ldb] : b[l + static_cast<size_t>(j) * ldb]; };
-  std::vector<float> acc(static_cast<size_t>(m) * 4);
-  constexpr int kBlockK = 256;
-  for (int j0 = 0; j0 < n; j0 += 4) {
-    const int nj = std::min(4, n - j0);
-    std::fill(acc.begin(), acc.end(), 0.f);
-    float* c0 = acc.data();
-    float* c1 = c0 + m;
-    float* c2 = c1 + m;
-    float* c3 = c2 + m;
-    float* cols[4] = {c0, c1, c2, c3};
-    if (!ta) {
-      for (int l0 = 0; l0 < k; l0 += kBlockK) {
-        const int l1 = std::min(k, l0 + kBlockK);
-        for (int l = l0; l < l1; ++l) {
-          const float* al = a + static_cast<size_t>(l) * lda;
-          if (nj == 4) {
-            const float b0 = b_at(l, j0), b1 = b_at(l, j0 + 1), b2 = b_at(l, j0 + 2), b3 = b_at(l, j0 + 3);
-            for (int i = 0; i < m; ++i) {
-              const float v = al[i];
-              c0[i] += v * b0;
-              c1[i] += v * b1;
-              c2[i] += v * b2;
-              c3[i] += v * b3;
-            }
-          } else {
-            for (int jj = 0; jj < nj; ++jj) {
-              const float bv = b_at(l, j0 + jj);
-              float* c = cols[jj];
-              for (int i = 0; i < m; ++i) c[i] += al[i] * bv;
-            }
-          }
-        }
-      }
-    } else {
-      // op(A)(i, l) = A(l, i): column i of the stored A against column j of op(B)
-      std::vector<float> bcol(static_cast<size_t>(k));
-      for (int jj = 0; jj < nj; ++jj) {
-        for (int l = 0; l < k; ++l) bcol[l] = b_at(l, j0 + jj);
-        float* c = cols[jj];
-        for (int i = 0; i < m; ++i) {
-          const float* ai = a + static_cast<size_t>(i) * lda;
-          float s = 0.f;
-          for (int l = 0; l < k; ++l) s += ai[l] * bcol[l];
-          c[i] = s;
-        }
-      }
-    }
-    for (int jj = 0; jj < nj; ++jj) {
-      S* out = C + static_cast<size_t>(j0 + jj) * ldc;
-      const float* c = cols[jj];
-      if (beta != 0.f)
-        for (int i = 0; i < m; ++i) put(out, i, c[i] + beta * get(out, i));
-      else
-        for (int i = 0; i < m; ++i) put(out, i, c[i]);
-    }
+  // the product alone in fp32: in C itself when C is fp32 and overwritten, else in a buffer of its own
+  const bool in_place = std::is_same_v<S, float> && beta == 0.f;
+  std::vector<float> sums(in_place ? 0 : static_cast<size_t>(m) * n);
+  float* c = in_place ? reinterpret_cast<float*>(C) : sums.data();
+  const int ldsum = in_place ? ldc : m;
+  if (k <= 0) {
+    for (int j = 0; j < n; ++j) std::fill(c + static_cast<size_t>(j) * ldsum, c + static_cast<size_t>(j) * ldsum + m, 0.f);
+  } else if (n < kNr || m < kMr || static_cast<double>(m) * n * k < 32768.) {
+    gemm_sweep(ta, tb, m, n, k, a, lda, b, ldb, c, ldsum);
+  } else {
+    gemm_packed(ta, tb, m, n, k, a, lda, b, ldb, c, ldsum);
+  }
+  if (in_place) return;
+  for (int j = 0; j < n; ++j) {
+    S* out = C + static_cast<size_t>(j) * ldc;
+    const float* cj = sums.data() + static_cast<size_t>(j) * m;
+    if (beta != 0.f)
+      for (int i = 0; i < m; ++i) put(out, static_cast<size_t>(i), cj[i] + beta * get(out, static_cast<size_t>(i)));
+    else
+      for (int i = 0; i < m; ++i) put(out, static_cast<size_t>(i), cj[i]);
   }
 }
 
