@@ -549,6 +549,21 @@ def bench_gpt(iters, cpu, dtype="bf16", executor=6, train=None):
         p = N.GptBlockParams(**params)
         r["cpu_ms"] = round(_cpu_timed(lambda: N.gpt_layer_forward_backward(p, x, targets, nh)), 1)
         r["cpu"] = "oracle (numpy fp32 restatement, BLAS products), 1 thread"
+        # The same graph with its nodes on cpu(), in fp32 as the reference's CPU device runs it: node by node
+        # through the host layer's own loops, one pass after an untimed one.
+        ex.scenario_set_device(1)
+        try:
+            cms = ctypes.c_float(0)
+            rc = ex.scenario_gpt_layer(DT["f32"], C, nh, B, T, V, _fp(x),
+                                       targets.ctypes.data_as(ctypes.POINTER(ctypes.c_int)),
+                                       (FP * 20)(*map(_fp, pin)), 1, _fp(loss), (FP * 20)(*map(_fp, grads)), _fp(dx),
+                                       ctypes.byref(cms), ctypes.byref(nodes))
+        finally:
+            ex.scenario_set_device(0)
+        if rc:
+            raise SystemExit(ex.scenario_last_error().decode())
+        r["cpu_nodes_ms"] = round(cms.value, 1)
+        r["cpu_nodes"] = "the same graph on cpu() in fp32: host layer nodes, 1 thread"
     return r
 
 
@@ -624,6 +639,7 @@ def other_configs(h, cpu):
     out["gpt_ms"], out["gpt_tflops"] = g["gpu_ms"], g["tflops"]
     if cpu:
         out["gpt_cpu_ms"] = g["cpu_ms"]
+        out["gpt_cpu_nodes_ms"] = g["cpu_nodes_ms"]
     out["gpt_kernels_per_pass"] = bench_gpt(2, False, executor=14)["kernels_per_pass"]
     r = bench_mlp(100, cpu, executor=6)
     out["mlp_ms"], out["mlp_gbs"] = r["gpu_ms"], r["gbs"]
@@ -642,8 +658,9 @@ def other_configs(h, cpu):
                    "autobatched LSTM fp32 256 seqs; gbs = algorithmic bytes of the pass's products per second; "
                    "kernels_per_pass = kernel nodes of the pass recorded as a device graph; attention = fp16 batch 128 "
                    "products, skinny = M = K = 4096 NN with the split-K fold included, against 8 TB/s; squares "
-                   "against 2.5 PFLOP/s; cpu = numpy fp32 oracle on 1 thread; mlp_cpu_nodes_ms / lstm_cpu_nodes_ms = the same "
-                   "graph with its nodes on cpu() (the host layer's own fp32 loops, node by node, 1 thread)")
+                   "against 2.5 PFLOP/s; cpu = numpy fp32 oracle on 1 thread; gpt_cpu_nodes_ms / mlp_cpu_nodes_ms / "
+                   "lstm_cpu_nodes_ms = the same graph with its nodes on cpu() (the host layer's own fp32 loops and "
+                   "packed product, node by node, 1 thread)")
     return out
 
 

@@ -42,26 +42,53 @@ inline const float* as_f32(const S* src, size_t ld, size_t cols, std::vector<flo
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
 // C[m x n] = op(A)[m x k] * op(B)[k x n] + beta * C, column-major, fp32 accumulation, one rounding to S.
-// Narrow or small products: blocked over K (the panel of A that a column block of C reuses stays in cache) with
-// four columns of C per sweep over a column of A; a transposed A turns the sweep into dot products of
-// contiguous columns.
-inline void gemm_sweep(bool ta, bool tb, int m, int n, int k, const float* a, int lda, const float* b, int ldb,
-                       float* c, int ldc) {
+//
+// The inner loops are written on vectors of W floats (GCC / clang vector types) and exist twice: eight-wide with
+// fused multiply-adds, compiled for AVX2 + FMA and taken when the processor has both (asked once at run time:
+// the library itself is built for any x86-64), and four-wide for everything else.
+// ---------------------------------------------------------------------------------------------------------
+template <int W>
+struct Vec {
+  typedef float type __attribute__((vector_size(W * sizeof(float)), aligned(4)));
+};
+// Unaligned vector access through the pointer (V is the vector type in scope).
+#define GINN_VLD(p) (*reinterpret_cast<const V*>(p))
+#define GINN_VST(p, v) (*reinterpret_cast<V*>(p) = (v))
+// (A float operand beside a vector is spread over the lanes by the compiler.)
+
+// Narrow or small products.  Without a transposed A: up to four columns of C per sweep over a column of A
+// (c_j += a_l * b(l, j)).  With one: dot products of contiguous columns, W partial sums each.
+template <int W>
+__attribute__((always_inline)) inline void sweep_impl(bool ta, bool tb, int m, int n, int k, const float* a, int lda,
+                                                      const float* b, int ldb, float beta, float* c, int ldc) {
+  using V = typename Vec<W>::type;
   auto b_at = [&](int l, int j) { return tb ? b[j + static_cast<size_t>(l) * ldb] : b[l + static_cast<size_t>(j) * ldb]; };
-  std::vector<float> bcol(ta ? static_cast<size_t>(k) : 0);
-  for (int j0 = 0; j0 < n; j0 += 4) {
-    const int nj = std::min(4, n - j0);
-    float* cols[4];
-    for (int jj = 0; jj < 4; ++jj) cols[jj] = c + static_cast<size_t>(j0 + std::min(jj, nj - 1)) * ldc;
-    for (int jj = 0; jj < nj; ++jj) std::fill(cols[jj], cols[jj] + m, 0.f);
-    if (!ta) {
+  if (!ta) {
+    for (int j0 = 0; j0 < n; j0 += 4) {
+      const int nj = std::min(4, n - j0);
+      float* cols[4];
+      for (int jj = 0; jj < 4; ++jj) cols[jj] = c + static_cast<size_t>(j0 + std::min(jj, nj - 1)) * ldc;
+      for (int jj = 0; jj < nj; ++jj) {
+        if (beta == 0.f) std::fill(cols[jj], cols[jj] + m, 0.f);
+        else if (beta != 1.f)
+          for (int i = 0; i < m; ++i) cols[jj][i] *= beta;
+      }
       for (int l = 0; l < k; ++l) {
         const float* al = a + static_cast<size_t>(l) * lda;
         if (nj == 4) {
           const float b0 = b_at(l, j0), b1 = b_at(l, j0 + 1), b2 = b_at(l, j0 + 2), b3 = b_at(l, j0 + 3);
           float *c0 = cols[0], *c1 = cols[1], *c2 = cols[2], *c3 = cols[3];
-          for (int i = 0; i < m; ++i) {
+          int i = 0;
+          for (; i + W <= m; i += W) {
+            const V av = GINN_VLD(al + i);
+            GINN_VST(c0 + i, GINN_VLD(c0 + i) + av * b0);
+            GINN_VST(c1 + i, GINN_VLD(c1 + i) + av * b1);
+            GINN_VST(c2 + i, GINN_VLD(c2 + i) + av * b2);
+            GINN_VST(c3 + i, GINN_VLD(c3 + i) + av * b3);
+          }
+          for (; i < m; ++i) {
             const float v = al[i];
             c0[i] += v * b0;
             c1[i] += v * b1;
@@ -70,23 +97,34 @@ inline void gemm_sweep(bool ta, bool tb, int m, int n, int k, const float* a, in
           }
         } else {
           for (int jj = 0; jj < nj; ++jj) {
-            const float bv = b_at(l, j0 + jj);
+            const float bs = b_at(l, j0 + jj);
             float* cj = cols[jj];
-            for (int i = 0; i < m; ++i) cj[i] += al[i] * bv;
+            int i = 0;
+            for (; i + W <= m; i += W) GINN_VST(cj + i, GINN_VLD(cj + i) + GINN_VLD(al + i) * bs);
+            for (; i < m; ++i) cj[i] += al[i] * bs;
           }
         }
       }
-    } else {
-      // op(A)(i, l) = A(l, i): column i of the stored A against column j of op(B)
-      for (int jj = 0; jj < nj; ++jj) {
-        for (int l = 0; l < k; ++l) bcol[static_cast<size_t>(l)] = b_at(l, j0 + jj);
-        float* cj = cols[jj];
-        for (int i = 0; i < m; ++i) {
-          const float* ai = a + static_cast<size_t>(i) * lda;
-          float sum = 0.f;
-          for (int l = 0; l < k; ++l) sum += ai[l] * bcol[static_cast<size_t>(l)];
-          cj[i] = sum;
-        }
+    }
+  } else {
+    // op(A)(i, l) = A(l, i): column i of the stored A against column j of op(B)
+    std::vector<float> bcol(tb ? static_cast<size_t>(k) : 0);
+    for (int j = 0; j < n; ++j) {
+      const float* bj = b + static_cast<size_t>(j) * ldb;
+      if (tb) {
+        for (int l = 0; l < k; ++l) bcol[static_cast<size_t>(l)] = b_at(l, j);
+        bj = bcol.data();
+      }
+      float* cj = c + static_cast<size_t>(j) * ldc;
+      for (int i = 0; i < m; ++i) {
+        const float* ai = a + static_cast<size_t>(i) * lda;
+        V acc = {};
+        int l = 0;
+        for (; l + W <= k; l += W) acc += GINN_VLD(ai + l) * GINN_VLD(bj + l);
+        float sum = 0.f;
+        for (int e = 0; e < W; ++e) sum += acc[e];
+        for (; l < k; ++l) sum += ai[l] * bj[l];
+        cj[i] = beta == 0.f ? sum : sum + beta * cj[i];
       }
     }
   }
@@ -95,54 +133,75 @@ inline void gemm_sweep(bool ta, bool tb, int m, int n, int k, const float* a, in
 // Everything else: the classic packed scheme.  op(A) is cut into blocks of kMc rows x kKc sums, stored as panels
 // of kMr rows (one sum after the other), op(B) into panels of kNr columns; a register tile of kMr x kNr sums runs
 // over one pair of panels.  Panels are padded with zeros, so the tile loop has no edges; edge tiles are stored
-// through a small buffer.  The tile loop exists twice: eight-wide with fused multiply-adds where the processor has
-// them (asked at run time: the library is built for any x86-64), and as plain loops.
+// through a small buffer.
 constexpr int kMr = 16, kNr = 6, kKc = 256, kMc = 128, kNc = 1536;
 
-// tile[j * kMr + i] = sum_l ap[l * kMr + i] * bp[l * kNr + j]
-inline void tile_plain(int kc, const float* ap, const float* bp, float* tile) {
-  float acc[kNr][kMr] = {};
-  for (int l = 0; l < kc; ++l, ap += kMr, bp += kNr)
-    for (int j = 0; j < kNr; ++j)
-      for (int i = 0; i < kMr; ++i) acc[j][i] += ap[i] * bp[j];
-  for (int j = 0; j < kNr; ++j)
-    for (int i = 0; i < kMr; ++i) tile[j * kMr + i] = acc[j][i];
-}
-#if defined(__x86_64__) && (defined(__GNUC__) || defined(__clang__))
-#define GINN_HOST_GEMM_HAS_FMA_TILE 1
-typedef float tile_v8 __attribute__((vector_size(32), aligned(4)));
-__attribute__((target("avx2,fma"))) inline void tile_fma(int kc, const float* ap, const float* bp, float* tile) {
-  tile_v8 acc[kNr][2] = {};
-  for (int l = 0; l < kc; ++l, ap += kMr, bp += kNr) {
-    const tile_v8 a0 = *reinterpret_cast<const tile_v8*>(ap);
-    const tile_v8 a1 = *reinterpret_cast<const tile_v8*>(ap + 8);
+// tile[j * kMr + i] = sum_l ap[l * kMr + i] * bp[l * kNr + j]; two vectors of rows per sweep, so that the
+// 2 x kNr sums stay in registers (four-wide: two sweeps of eight rows).
+template <int W>
+__attribute__((always_inline)) inline void tile_impl(int kc, const float* ap, const float* bp, float* tile) {
+  using V = typename Vec<W>::type;
+  for (int r0 = 0; r0 < kMr; r0 += 2 * W) {
+    V acc[kNr][2] = {};
+    const float* a = ap + r0;
+    const float* b = bp;
+    for (int l = 0; l < kc; ++l, a += kMr, b += kNr) {
+      const V a0 = GINN_VLD(a), a1 = GINN_VLD(a + W);
 #pragma GCC unroll 6
+      for (int j = 0; j < kNr; ++j) {
+        const float bj = b[j];
+        acc[j][0] += a0 * bj;
+        acc[j][1] += a1 * bj;
+      }
+    }
     for (int j = 0; j < kNr; ++j) {
-      const float bj = bp[j];
-      const tile_v8 bv = {bj, bj, bj, bj, bj, bj, bj, bj};
-      acc[j][0] += a0 * bv;
-      acc[j][1] += a1 * bv;
+      GINN_VST(tile + j * kMr + r0, acc[j][0]);
+      GINN_VST(tile + j * kMr + r0 + W, acc[j][1]);
     }
   }
-  for (int j = 0; j < kNr; ++j) {
-    *reinterpret_cast<tile_v8*>(tile + j * kMr) = acc[j][0];
-    *reinterpret_cast<tile_v8*>(tile + j * kMr + 8) = acc[j][1];
-  }
 }
-inline bool has_fma_tile() {
+
+inline void sweep_narrow(bool ta, bool tb, int m, int n, int k, const float* a, int lda, const float* b, int ldb,
+                         float beta, float* c, int ldc) {
+  sweep_impl<4>(ta, tb, m, n, k, a, lda, b, ldb, beta, c, ldc);
+}
+inline void tile_narrow(int kc, const float* ap, const float* bp, float* tile) { tile_impl<4>(kc, ap, bp, tile); }
+#if defined(__x86_64__) && (defined(__GNUC__) || defined(__clang__)) && !defined(GINN_HOST_GEMM_PLAIN)
+__attribute__((target("avx2,fma"))) inline void sweep_wide(bool ta, bool tb, int m, int n, int k, const float* a,
+                                                           int lda, const float* b, int ldb, float beta, float* c,
+                                                           int ldc) {
+  sweep_impl<8>(ta, tb, m, n, k, a, lda, b, ldb, beta, c, ldc);
+}
+__attribute__((target("avx2,fma"))) inline void tile_wide(int kc, const float* ap, const float* bp, float* tile) {
+  tile_impl<8>(kc, ap, bp, tile);
+}
+inline bool has_wide_vectors() {
   static const bool yes = __builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma");
   return yes;
 }
 #else
-inline void tile_fma(int kc, const float* ap, const float* bp, float* tile) { tile_plain(kc, ap, bp, tile); }
-inline bool has_fma_tile() { return false; }
+inline void sweep_wide(bool ta, bool tb, int m, int n, int k, const float* a, int lda, const float* b, int ldb,
+                       float beta, float* c, int ldc) {
+  sweep_narrow(ta, tb, m, n, k, a, lda, b, ldb, beta, c, ldc);
+}
+inline void tile_wide(int kc, const float* ap, const float* bp, float* tile) { tile_narrow(kc, ap, bp, tile); }
+inline bool has_wide_vectors() { return false; }
 #endif
 
-// c (fp32, leading dimension ldc) = op(a) op(b); c is overwritten.
+#undef GINN_VLD
+#undef GINN_VST
+
+// c (fp32, leading dimension ldc) = op(a) op(b) + beta * c
 inline void gemm_packed(bool ta, bool tb, int m, int n, int k, const float* a, int lda, const float* b, int ldb,
-                        float* c, int ldc) {
-  const bool fma = has_fma_tile();
-  std::vector<float> apack(static_cast<size_t>(kMc) * kKc), bpack(static_cast<size_t>(kKc) * (kNc + kNr));
+                        float beta, float* c, int ldc) {
+  const bool wide = has_wide_vectors();
+  // packed blocks, kept per thread between calls (a fresh 1.5 MB block per call costs more than a small product)
+  static thread_local std::vector<float> apack, bpack;
+  const size_t kc_max = static_cast<size_t>(std::min(k, kKc));
+  const size_t a_need = kc_max * static_cast<size_t>((std::min(m, kMc) + kMr - 1) / kMr * kMr);
+  const size_t b_need = kc_max * static_cast<size_t>((std::min(n, kNc) + kNr - 1) / kNr * kNr);
+  if (apack.size() < a_need) apack.resize(a_need);
+  if (bpack.size() < b_need) bpack.resize(b_need);
   float tile[kMr * kNr];
   for (int jc = 0; jc < n; jc += kNc) {
     const int nc = std::min(kNc, n - jc);
@@ -193,15 +252,19 @@ inline void gemm_packed(bool ta, bool tb, int m, int n, int k, const float* a, i
           for (int i0 = 0; i0 < mc; i0 += kMr) {
             const int mr = std::min(kMr, mc - i0);
             const float* ap = apack.data() + static_cast<size_t>(i0) * kc;
-            if (fma) tile_fma(kc, ap, bp, tile);
-            else tile_plain(kc, ap, bp, tile);
+            if (wide) tile_wide(kc, ap, bp, tile);
+            else tile_narrow(kc, ap, bp, tile);
             float* out = c + (ic + i0) + static_cast<size_t>(jc + j0) * ldc;
-            if (pc == 0) {
+            if (pc == 0 && beta == 0.f) {
               for (int j = 0; j < nr; ++j)
                 for (int i = 0; i < mr; ++i) out[i + static_cast<size_t>(j) * ldc] = tile[j * kMr + i];
             } else {
+              const float scale = pc == 0 ? beta : 1.f;
               for (int j = 0; j < nr; ++j)
-                for (int i = 0; i < mr; ++i) out[i + static_cast<size_t>(j) * ldc] += tile[j * kMr + i];
+                for (int i = 0; i < mr; ++i) {
+                  float& o = out[i + static_cast<size_t>(j) * ldc];
+                  o = scale * o + tile[j * kMr + i];
+                }
             }
           }
         }
@@ -217,17 +280,17 @@ void gemm(bool ta, bool tb, int m, int n, int k, const S* A, int lda, const S* B
   std::vector<float> keep_a, keep_b;
   const float* a = as_f32(A, static_cast<size_t>(lda), static_cast<size_t>(ta ? m : k), keep_a);
   const float* b = as_f32(B, static_cast<size_t>(ldb), static_cast<size_t>(tb ? k : n), keep_b);
-  // the product alone in fp32: in C itself when C is fp32 and overwritten, else in a buffer of its own
-  const bool in_place = std::is_same_v<S, float> && beta == 0.f;
+  // fp32 results form in C itself; the 16-bit types get the product alone in fp32 first and one rounding after
+  constexpr bool in_place = std::is_same_v<S, float>;
   std::vector<float> sums(in_place ? 0 : static_cast<size_t>(m) * n);
   float* c = in_place ? reinterpret_cast<float*>(C) : sums.data();
   const int ldsum = in_place ? ldc : m;
-  if (k <= 0) {
-    for (int j = 0; j < n; ++j) std::fill(c + static_cast<size_t>(j) * ldsum, c + static_cast<size_t>(j) * ldsum + m, 0.f);
-  } else if (n < kNr || m < kMr || static_cast<double>(m) * n * k < 32768.) {
-    gemm_sweep(ta, tb, m, n, k, a, lda, b, ldb, c, ldsum);
+  const float inner_beta = in_place ? beta : 0.f;
+  if (n < kNr || m < kMr || k < 8 || static_cast<double>(m) * n * k < 32768.) {
+    if (has_wide_vectors()) sweep_wide(ta, tb, m, n, k, a, lda, b, ldb, inner_beta, c, ldsum);
+    else sweep_narrow(ta, tb, m, n, k, a, lda, b, ldb, inner_beta, c, ldsum);
   } else {
-    gemm_packed(ta, tb, m, n, k, a, lda, b, ldb, c, ldsum);
+    gemm_packed(ta, tb, m, n, k, a, lda, b, ldb, inner_beta, c, ldsum);
   }
   if (in_place) return;
   for (int j = 0; j < n; ++j) {

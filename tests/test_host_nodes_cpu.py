@@ -28,6 +28,8 @@ def cpu_shim():
 @pytest.mark.parametrize("dt", G.DTYPES)
 @pytest.mark.parametrize("a_shape,b_shape,batched", [
     ((2, 3), (3, 2), 0), ((64, 48), (48, 33), 0), ((130, 70), (70, 96), 0), ((4, 6, 5), (30, 7), 0),
+    # the packed product's edges: rows and columns that fill no register tile, sums across two K blocks
+    ((37, 53), (53, 29), 0), ((300, 260), (260, 23), 0), ((17, 600), (600, 135), 0),
     ((2, 3, 4), (3, 5, 4), 1), ((2, 3, 2, 2), (3, 5, 2, 2), 1), ((64, 32, 8), (32, 48, 8), 1)])
 def test_prod_nodes_on_cpu(cpu_shim, dt, a_shape, b_shape, batched):
     G.test_prod_nodes(cpu_shim, dt, a_shape, b_shape, batched)
