@@ -111,6 +111,22 @@ int launch_gemm_mid(ginn_hip_ctx* ctx, const GemmArgs& a) {
   const long long tiles = (long long)p.tiles_m * p.tiles_n;
   p.group = (tiles % 8 == 0) ? 8 : 0;
   if (p.group > p.tiles_m) p.group = p.tiles_m;
+  // Few tiles per XCD: make an XCD's share an exact block of g tile rows x (share / g) tile columns with the
+  // smallest g + share / g, the operand panels its L2 has to fetch (12 x 12 tiles of 64 x 64 over K = 4096:
+  // blocks of 6 x 3 instead of 8 rows x 2.25 columns, 16.2 -> 14.0 us; nothing changes for the other shapes
+  // measured).  Larger outputs keep panels of 8 rows.
+  if (p.group > 0 && tiles / 8 <= 32) {
+    const int per = (int)(tiles / 8);
+    int best = 0, cost = 1 << 30;
+    for (int g = 1; g <= p.tiles_m && g <= per; ++g) {
+      if (per % g || p.tiles_m % g || p.tiles_n % (per / g)) continue;
+      if (g + per / g <= cost) {
+        best = g;
+        cost = g + per / g;
+      }
+    }
+    if (best) p.group = best;
+  }
   const bool akc = a.op_a == GINN_HIP_OP_T;
   const bool bkc = a.op_b == GINN_HIP_OP_N;
   const int kt_total = (a.k + bk - 1) / bk;
