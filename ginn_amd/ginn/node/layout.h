@@ -698,7 +698,6 @@ class ChipNode : public BaseDataNode<Scalar> {
     for (size_t a = static_cast<size_t>(dim_) + 1; a < s.size(); ++a) outer *= s[a];
   }
   void forward_() override {
-    internal::require_gpu(this->dev(), "Chip");
     const Shape in_s = in_->shape();
     GINN_ASSERT(dim_ >= 0 && static_cast<size_t>(dim_) < in_s.size());
     GINN_ASSERT(offset_ >= 0 && offset_ < in_s[static_cast<size_t>(dim_)]);
@@ -708,18 +707,14 @@ class ChipNode : public BaseDataNode<Scalar> {
     value().resize(s);
     Size inner, extent, outer;
     geometry(inner, extent, outer);
-    GINN_HIP_CALL(ginn_hip_copy_2d(internal::ctx_of(value()), internal::move_dtype_of<Scalar>(), static_cast<int>(inner),
-                                   static_cast<int>(outer), in_->value().data() + offset_ * inner,
-                                   static_cast<int>(inner * extent), value().data(), static_cast<int>(inner), 0));
+    internal::copy_2d(value(), 0, inner, in_->value(), offset_ * inner, inner * extent, inner, outer, false);
   }
   void backward_() override {
     if (!in_->has_grad()) return;
     if constexpr (is_floating_point_v<Scalar>) {
       Size inner, extent, outer;
       geometry(inner, extent, outer);
-      GINN_HIP_CALL(ginn_hip_copy_2d(internal::ctx_of(grad()), dtype_of<Scalar>(), static_cast<int>(inner),
-                                     static_cast<int>(outer), grad().data(), static_cast<int>(inner),
-                                     in_->grad().data() + offset_ * inner, static_cast<int>(inner * extent), 1));
+      internal::copy_2d(in_->grad(), offset_ * inner, inner * extent, grad(), 0, inner, inner, outer, true);
     }
   }
 

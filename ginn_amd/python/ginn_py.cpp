@@ -118,11 +118,30 @@ void from_numpy(Tensor<S>& t, const py::array& any) {
 
 template <typename S>
 void bind_tensor(py::module_& m) {
+  // values as Python hands them over (numbers or bools), converted to the tensor's scalar
+  using Host = std::conditional_t<is_floating_point_v<S>, float, S>;
+  auto with_values = [](const DevPtr& dev, const Shape& shape, const std::vector<Host>& val) {
+    Tensor<S> t(dev, shape);
+    std::vector<S> v(val.size());
+    for (size_t i = 0; i < v.size(); ++i) v[i] = S(val[i]);
+    t.set(v);
+    return t;
+  };
+  // the constructors of ginn-py/tensor-py.cu.cpp:36-45
   py::class_<Tensor<S>>(m, named<S>("Tensor").c_str())
-      .def(py::init([](const DevPtr& dev, const Shape& shape) { return Tensor<S>(dev, shape); }), py::arg("dev"),
+      .def(py::init([]() { return Tensor<S>(cpu(), Shape{0}); }))
+      .def(py::init([](const DevPtr& dev) { return Tensor<S>(dev, Shape{0}); }), py::arg("device"))
+      .def(py::init([](const Shape& shape) { return Tensor<S>(cpu(), shape); }), py::arg("shape"))
+      .def(py::init([with_values](const Shape& shape, const std::vector<Host>& val) {
+             return with_values(cpu(), shape, val);
+           }),
+           py::arg("shape"), py::arg("val"))
+      .def(py::init([](const DevPtr& dev, const Shape& shape) { return Tensor<S>(dev, shape); }), py::arg("device"),
            py::arg("shape"))
+      .def(py::init(with_values), py::arg("device"), py::arg("shape"), py::arg("val"))
       .def_property_readonly("dev", [](const Tensor<S>& t) { return t.dev(); })
-      .def_property_readonly("shape", [](const Tensor<S>& t) { return t.shape(); })
+      .def_property("shape", [](const Tensor<S>& t) { return t.shape(); },
+                    [](Tensor<S>& t, const Shape& shape) { t.resize(shape); })
       .def_property_readonly("size", [](const Tensor<S>& t) { return t.size(); })
       .def_property_readonly("scalar", [](const Tensor<S>&) {
         if constexpr (std::is_same_v<S, Real>) return Scalar_::Real;
@@ -132,24 +151,69 @@ void bind_tensor(py::module_& m) {
         else return Scalar_::Bool;
       })
       .def("numpy", &to_numpy<S>)
-      .def("m", [](const Tensor<S>& t) {
+      // m() / v(): the tensor as a matrix / vector.  Real and Int tensors on cpu() hand out a view of their own
+      // memory that writes through, like the Eigen maps of ginn-py (ginn-py/test/test_tensor.py:114-127); the
+      // other scalars and device tensors hand out a copy.
+      .def("m", [](py::object self) -> py::object {
+        Tensor<S>& t = self.cast<Tensor<S>&>();
+        if constexpr (std::is_same_v<S, Real> || std::is_same_v<S, Int>) {
+          if (t.dev()->kind() == CPU && t.size() > 0)
+            return py::array_t<S>({static_cast<py::ssize_t>(t.rows()), static_cast<py::ssize_t>(t.cols())},
+                                  {static_cast<py::ssize_t>(sizeof(S)), static_cast<py::ssize_t>(sizeof(S) * t.rows())},
+                                  t.data(), self);
+        }
         return to_numpy(t).attr("reshape")(py::make_tuple(t.rows(), t.cols()), py::arg("order") = "F");
       })
-      .def("v", [](const Tensor<S>& t) { return to_numpy(t).attr("reshape")(py::make_tuple(-1), py::arg("order") = "F"); })
+      .def("v", [](py::object self) -> py::object {
+        Tensor<S>& t = self.cast<Tensor<S>&>();
+        if constexpr (std::is_same_v<S, Real> || std::is_same_v<S, Int>) {
+          if (t.dev()->kind() == CPU && t.size() > 0)
+            return py::array_t<S>({static_cast<py::ssize_t>(t.size())}, {static_cast<py::ssize_t>(sizeof(S))}, t.data(),
+                                  self);
+        }
+        return to_numpy(t).attr("reshape")(py::make_tuple(-1), py::arg("order") = "F");
+      })
       .def("list", [](const Tensor<S>& t) {
         using Out = std::conditional_t<is_floating_point_v<S>, float, S>;
         std::vector<Out> out;
         for (const S& x : t.vector()) out.push_back(static_cast<Out>(x));
         return out;
       })
-      .def("set", &from_numpy<S>)
+      // an array or nested lists: [[1, 2, 3], [4, 5, 6]] is a 2 x 3 tensor (ginn/tensor.h:331-395)
+      .def("set", [](Tensor<S>& t, const py::object& values) {
+        auto a = py::array::ensure(values);
+        if (!a) throw std::invalid_argument("set() takes an array or nested lists of numbers");
+        from_numpy<S>(t, a);
+      })
+      .def("item", [](const Tensor<S>& t) { return static_cast<std::conditional_t<is_floating_point_v<S>, float, S>>(t.item()); })
+      .def("real", [](const Tensor<S>& t) { return t.template cast<Real>(); })
+      .def("half", [](const Tensor<S>& t) { return t.template cast<Half>(); })
+      .def("bfloat16", [](const Tensor<S>& t) { return t.template cast<BFloat16>(); })
+      .def("int", [](const Tensor<S>& t) { return t.template cast<Int>(); })
+      .def("bool", [](const Tensor<S>& t) { return t.template cast<bool>(); })
+      .def("cast",
+           [](const Tensor<S>& t, Scalar_ s) -> py::object {
+             switch (s) {
+               case Scalar_::Real: return py::cast(t.template cast<Real>());
+               case Scalar_::Half: return py::cast(t.template cast<Half>());
+               case Scalar_::BFloat16: return py::cast(t.template cast<BFloat16>());
+               case Scalar_::Int: return py::cast(t.template cast<Int>());
+               default: return py::cast(t.template cast<bool>());
+             }
+           })
+      .def("set_ones", [](Tensor<S>& t) { t.set_ones(); })
       .def("set_zero", [](Tensor<S>& t) { t.set_zero(); })
       .def("set_random", [](Tensor<S>& t) { t.set_random(); })
-      .def("fill", [](Tensor<S>& t, double v) { t.fill(S(static_cast<float>(v))); })
-      .def("move_to", [](Tensor<S>& t, const DevPtr& dev) { t.move_to(dev); })
+      .def("fill", [](Tensor<S>& t, double v) { t.fill(S(static_cast<float>(v))); }, py::arg("val"))
+      .def("move_to", [](Tensor<S>& t, const DevPtr& dev) { t.move_to(dev); }, py::arg("device"))
       .def("copy_to", [](const Tensor<S>& t, const DevPtr& dev) { return t.copy_to(dev); })
       .def("maybe_copy_to", [](Tensor<S>& t, const DevPtr& dev) { return t.maybe_copy_to(dev); })
-      .def("__eq__", [](const Tensor<S>& a, const Tensor<S>& b) { return a == b; })
+      .def("__eq__", [](const Tensor<S>& a, const Tensor<S>& b) { return a == b; }, py::is_operator())
+      .def("__repr__", [](const Tensor<S>& t) {
+        std::ostringstream out;
+        t.save(out);
+        return out.str();
+      })
       // the text form of Tensor::save / load
       .def("dumps", [](const Tensor<S>& t) {
         std::ostringstream out;
@@ -198,16 +262,17 @@ void bind_node_types(py::module_& m) {
             else throw std::invalid_argument("has_grad cannot be set on this node");
           });
   auto data = py::class_<DataNode<S>, N, SP<DataNode<S>>>(m, named<S>("DataNode").c_str());
-  data.def("move_to", [](DataNode<S>& n, const DevPtr& dev) { n.move_to(dev); })
+  data.def("move_to", [](DataNode<S>& n, const DevPtr& dev) { n.move_to(dev); }, py::arg("device"))
       .def("set_random", [](DataNode<S>& n) { n.set_random(); })
-      .def("fill", [](DataNode<S>& n, double v) { n.fill(S(static_cast<float>(v))); });
+      .def("fill", [](DataNode<S>& n, double v) { n.fill(S(static_cast<float>(v))); }, py::arg("val"));
   if constexpr (is_floating_point_v<S>) {
     py::class_<WeightNode<S>, N, SP<WeightNode<S>>>(m, named<S>("WeightNode").c_str())
         .def_property_readonly("id", &WeightNode<S>::id)
-        .def("move_to", [](WeightNode<S>& n, const DevPtr& dev) { n.move_to(dev); })
+        .def("move_to", [](WeightNode<S>& n, const DevPtr& dev) { n.move_to(dev); }, py::arg("device"))
         .def("set_random", [](WeightNode<S>& n) { n.value().set_random(); })
         .def("reset_grad", [](WeightNode<S>& n) { n.reset_grad(); })
-        .def("copy", [](WeightNode<S>& n, Copy mode) { return SP<WeightNode<S>>(n.copy(mode).as_shared_ptr()); });
+        .def("copy", [](WeightNode<S>& n, Copy mode) { return SP<WeightNode<S>>(n.copy(mode).as_shared_ptr()); },
+             py::arg("mode"));
   }
 }
 
@@ -225,14 +290,16 @@ void bind_shared_nodes(py::module_& m) {
   m.def("CwiseMax", [](const std::vector<SP<N>>& ins) { return as_node(CwiseMax(ptrs<S>(ins))); });
   m.def("CwiseProdAdd",
         [P](In a, In b, In c, double bias) { return as_node(CwiseProdAdd(P(a), P(b), P(c), S(static_cast<float>(bias)))); },
-        py::arg("a"), py::arg("b"), py::arg("c"), py::arg("multiplier_bias") = 0.);
+        py::arg("in"), py::arg("multiplicand"), py::arg("addend"), py::arg("multiplicand_bias") = 0.);
   m.def("AddScalar", [P](In x, double s) { return as_node(AddScalar(P(x), s)); });
   m.def("SubtractScalar", [P](double s, In x) { return as_node(SubtractScalar(s, P(x))); });
   m.def("ProdScalar", [P](In x, double s) { return as_node(ProdScalar(P(x), s)); });
-  m.def("Chip", [P](In x, Size offset, Size dim) { return as_node(Chip(P(x), offset, dim)); });
-  m.def("Reshape", [P](In x, const Shape& s) { return as_node(Reshape(P(x), s)); });
+  m.def("Chip", [P](In x, Size offset, Size dim) { return as_node(Chip(P(x), offset, dim)); }, py::arg("in"),
+        py::arg("offset"), py::arg("dim"));
+  m.def("Reshape", [P](In x, const Shape& s) { return as_node(Reshape(P(x), s)); }, py::arg("in"), py::arg("shape"));
   m.def("RankView", [P](In x, Size rank) { return as_node(RankView(P(x), rank)); }, py::arg("in"), py::arg("rank"));
-  m.def("Slice", [P](In x, const Shape& offsets, const Shape& sizes) { return as_node(Slice(P(x), offsets, sizes)); });
+  m.def("Slice", [P](In x, const Shape& offsets, const Shape& sizes) { return as_node(Slice(P(x), offsets, sizes)); },
+        py::arg("in"), py::arg("offsets"), py::arg("sizes"));
   m.def("Cat", [](const std::vector<SP<N>>& ins) { return as_node(Cat(ptrs<S>(ins))); });
   m.def("RowwiseCat", [](const std::vector<SP<N>>& ins) { return as_node(RowwiseCat(ptrs<S>(ins))); });
   m.def("Stack", [](const std::vector<std::vector<SP<N>>>& grid) {
@@ -241,10 +308,15 @@ void bind_shared_nodes(py::module_& m) {
     return as_node(Stack<S>(g));
   });
   m.def("LessThan", [P](In a, In b) { return SP<Node<bool>>(LessThan(P(a), P(b)).as_shared_ptr()); });
-  m.def("Permute", [P](In x, const Shape& s) { return as_node(Permute(P(x), s)); });
-  m.def("Transpose", [P](In x, Size i, Size j) { return as_node(Transpose(P(x), i, j)); });
-  m.def("RowBroadcast", [P](In x, Size rows) { return as_node(RowBroadcast(P(x), rows)); });
-  m.def("ColBroadcast", [P](In x, Size cols) { return as_node(ColBroadcast(P(x), cols)); });
+  m.def("Permute", [P](In x, const Shape& s) { return as_node(Permute(P(x), s)); }, py::arg("in"), py::arg("indices"));
+  m.def("Transpose", [P](In x, Size i, Size j) { return as_node(Transpose(P(x), i, j)); }, py::arg("in"), py::arg("i"),
+        py::arg("j"));
+  m.def("RowBroadcast", [P](In x, Size rows) { return as_node(RowBroadcast(P(x), rows)); }, py::arg("in"), py::arg("size"));
+  m.def("ColBroadcast", [P](In x, Size cols) { return as_node(ColBroadcast(P(x), cols)); }, py::arg("in"), py::arg("size"));
+  m.def("RowBroadcast", [P](In x, const SP<DimNode>& rows) { return as_node(RowBroadcast(P(x), DimPtr(rows))); },
+        py::arg("in"), py::arg("size"));
+  m.def("ColBroadcast", [P](In x, const SP<DimNode>& cols) { return as_node(ColBroadcast(P(x), DimPtr(cols))); },
+        py::arg("in"), py::arg("size"));
   m.def("Mask", [P](In x, In mask, double val) { return as_node(Mask(P(x), P(mask), val)); });
   m.def("Select", [P](const SP<Node<bool>>& c, In a, In b) { return as_node(Select(NodePtr<bool>(c), P(a), P(b))); });
   m.def("Select", [P](const SP<Node<bool>>& c, In a, double b) {
@@ -384,19 +456,40 @@ PYBIND11_MODULE(ginn, m) {
 
   // ---- devices (ginn-py/dev-py.cu.cpp) ----
   py::enum_<DeviceKind>(m, "DeviceKind").value("CPU", CPU).value("GPU", GPU).value("NULL_DEV", NULL_DEV);
+  m.attr("DeviceType") = m.attr("DeviceKind");  // the reference's name of the enumeration
+  py::class_<DeviceId>(m, "DeviceId")
+      .def_readonly("kind", &DeviceId::kind)
+      .def_readonly("idx", &DeviceId::idx)
+      .def("__repr__",
+           [](const DeviceId& i) {
+             return std::string("<DeviceId with kind: ") + (i.kind == CPU ? "CPU" : i.kind == GPU ? "GPU" : "NULL_DEV") +
+                    ", idx: " + std::to_string(i.idx) + ">";
+           })
+      .def("__eq__", [](const DeviceId& a, const DeviceId& b) { return a == b; }, py::is_operator());
+  // Devices compare by identity, as in ginn-py (no __eq__ there): cpu() and gpu(i) hand out one object each,
+  // Cpu() / Gpu(i) / the arenas a new one per call; ids compare by value.
   py::class_<Device, SP<Device>>(m, "Device")
       .def_property_readonly("kind", &Device::kind)
+      .def_property_readonly("id", &Device::id)
       .def_property_readonly("idx", [](const Device& d) { return d.id().idx; })
-      .def_property_readonly("precedence", &Device::precedence)
-      .def("__eq__", [](const Device& a, const Device& b) { return a.id() == b.id(); });
+      .def_property_readonly("precedence", &Device::precedence);
+  py::class_<PreallocCpuDevice, Device, SP<PreallocCpuDevice>>(m, "PreallocCpuDevice")
+      .def("clear", &PreallocCpuDevice::clear)
+      .def_property_readonly("used", &PreallocCpuDevice::used)
+      .def_property_readonly("size", &PreallocCpuDevice::size);
   py::class_<PreallocGpuDevice, Device, SP<PreallocGpuDevice>>(m, "PreallocGpuDevice")
       .def("clear", &PreallocGpuDevice::clear)
       .def_property_readonly("used", &PreallocGpuDevice::used)
       .def_property_readonly("size", &PreallocGpuDevice::size);
   m.def("cpu", []() -> SP<Device> { return cpu(); });
-  m.def("gpu", [](int idx) -> SP<Device> { return gpu(idx); }, py::arg("idx") = 0);
+  m.def("Cpu", []() -> SP<Device> { return Cpu(); });
+  m.def("gpu", [](int idx) -> SP<Device> { return gpu(idx); }, py::arg("gpu_idx") = 0);
+  m.def("Gpu", [](size_t idx) -> SP<Device> { return Gpu(idx); }, py::arg("gpu_idx") = 0);
   m.def("gpus", &gpus);
-  m.def("PreallocGpu", [](size_t bytes) { return PreallocGpu(bytes); });
+  m.def("PreallocCpu", [](size_t bytes) { return PreallocCpu(bytes); }, py::arg("size"));
+  m.def("PreallocGpu", [](size_t bytes) { return PreallocGpu(bytes); }, py::arg("size"));
+  m.def("PreallocGpu", [](size_t idx, size_t bytes) { return PreallocGpu(idx, bytes); }, py::arg("idx"),
+        py::arg("size"));
 
   // ---- tensors (ginn-py/tensor-py.cu.cpp) ----
   bind_tensor<Real>(m);
@@ -404,6 +497,22 @@ PYBIND11_MODULE(ginn, m) {
   bind_tensor<BFloat16>(m);
   bind_tensor<Int>(m);
   bind_tensor<bool>(m);
+  // Tensor(device, shape, scalar): the tensor class by scalar (ginn-py/tensor-py.cu.cpp:120-135)
+  auto tensor_of = [](const DevPtr& dev, const Shape& shape, Scalar_ s) -> py::object {
+    switch (s) {
+      case Scalar_::Real: return py::cast(Tensor<Real>(dev, shape));
+      case Scalar_::Half: return py::cast(Tensor<Half>(dev, shape));
+      case Scalar_::BFloat16: return py::cast(Tensor<BFloat16>(dev, shape));
+      case Scalar_::Int: return py::cast(Tensor<Int>(dev, shape));
+      default: return py::cast(Tensor<bool>(dev, shape));
+    }
+  };
+  m.def("Tensor", [tensor_of](Scalar_ s) { return tensor_of(cpu(), Shape{0}, s); }, py::arg("scalar") = Scalar_::Real);
+  m.def("Tensor", [tensor_of](const DevPtr& dev, Scalar_ s) { return tensor_of(dev, Shape{0}, s); }, py::arg("device"),
+        py::arg("scalar") = Scalar_::Real);
+  m.def("Tensor", tensor_of, py::arg("device"), py::arg("shape"), py::arg("scalar") = Scalar_::Real);
+  m.def("Tensor", [tensor_of](const Shape& shape, Scalar_ s) { return tensor_of(cpu(), shape, s); }, py::arg("shape"),
+        py::arg("scalar") = Scalar_::Real);
 
   // ---- nodes (ginn-py/node-py.cu.cpp) ----
   py::class_<BaseNode, SP<BaseNode>>(m, "BaseNode")
@@ -458,7 +567,23 @@ PYBIND11_MODULE(ginn, m) {
     n->set_has_grad(false);
     return SP<DataNode<Real>>(n.as_shared_ptr());
   });
-  m.def("Data", &data_node, py::arg("dev"), py::arg("shape"), py::arg("scalar") = Scalar_::Real);
+  // Data(device, scalar), Data(device, shape, scalar), Data(shape, scalar) (ginn-py/node-py.cu.cpp:190-196)
+  m.def("Data", &data_node, py::arg("device"), py::arg("shape"), py::arg("scalar") = Scalar_::Real);
+  m.def("Data", [](const DevPtr& dev, Scalar_ s) { return data_node(dev, Shape{0}, s); }, py::arg("device"),
+        py::arg("scalar") = Scalar_::Real);
+  m.def("Data", [](const Shape& shape, Scalar_ s) { return data_node(cpu(), shape, s); }, py::arg("shape"),
+        py::arg("scalar") = Scalar_::Real);
+  // RealData(dev, shape), HalfData, ... (ginn-py/node-py.cu.cpp:181-188)
+  m.def("RealData", [](const DevPtr& d, const Shape& s) { return data_node(d, s, Scalar_::Real); }, py::arg("dev"), py::arg("shape"));
+  m.def("HalfData", [](const DevPtr& d, const Shape& s) { return data_node(d, s, Scalar_::Half); }, py::arg("dev"), py::arg("shape"));
+  m.def("BFloat16Data", [](const DevPtr& d, const Shape& s) { return data_node(d, s, Scalar_::BFloat16); }, py::arg("dev"), py::arg("shape"));
+  m.def("IntData", [](const DevPtr& d, const Shape& s) { return data_node(d, s, Scalar_::Int); }, py::arg("dev"), py::arg("shape"));
+  m.def("BoolData", [](const DevPtr& d, const Shape& s) { return data_node(d, s, Scalar_::Bool); }, py::arg("dev"), py::arg("shape"));
+  // lazily evaluated sizes (ginn-py/node/layout-py.cu.cpp:128-131)
+  py::class_<DimNode, BaseNode, SP<DimNode>>(m, "DimNode").def_property_readonly("value", [](DimNode& d) { return d.value(); });
+  m.def("Dim", [](Size n) { return SP<DimNode>(Dim(n).as_shared_ptr()); }, py::arg("dims"));
+  m.def("Dim", [](const SP<BaseNode>& in, Size i) { return SP<DimNode>(Dim(BaseNodePtr(in), i).as_shared_ptr()); },
+        py::arg("in"), py::arg("dim_idx"));
   // UpperTri(dev, size, scalar) (ginn-py/node/layout-py.cu.cpp:30-46,113-125)
   m.def("UpperTri",
         [](const DevPtr& dev, Size size, Scalar_ s) -> py::object {
@@ -480,11 +605,22 @@ PYBIND11_MODULE(ginn, m) {
     if (arr.ndim() == 0) n->value().resize(Shape{});
     n->move_to(dev);
     return SP<DataNode<Real>>(n.as_shared_ptr());
-  });
-  m.def("Values", [](const py::object& nested) { return py::module_::import("ginn").attr("Values")(cpu(), nested); });
-  m.def("Random", [](const DevPtr& dev, const Shape& shape) {
-    return SP<DataNode<Real>>(Random<Real>(dev, shape).as_shared_ptr());
-  });
+  }, py::arg("dev"), py::arg("values"));
+  m.def("Values", [](const py::object& nested) {
+    return py::module_::import("ginn").attr("Values")(SP<Device>(cpu()), nested);
+  }, py::arg("values"));
+  // Random(device, shape, scalar), Random(shape, scalar): uniform in [-1, 1] (ginn-py/node-py.cu.cpp:203-209)
+  auto random_of = [](const DevPtr& dev, const Shape& shape, Scalar_ s) -> py::object {
+    switch (s) {
+      case Scalar_::Real: return py::cast(SP<DataNode<Real>>(Random<Real>(dev, shape).as_shared_ptr()));
+      case Scalar_::Half: return py::cast(SP<DataNode<Half>>(Random<Half>(dev, shape).as_shared_ptr()));
+      case Scalar_::BFloat16: return py::cast(SP<DataNode<BFloat16>>(Random<BFloat16>(dev, shape).as_shared_ptr()));
+      default: throw std::invalid_argument("Random: a floating-point scalar is needed");
+    }
+  };
+  m.def("Random", random_of, py::arg("device"), py::arg("shape"), py::arg("scalar") = Scalar_::Real);
+  m.def("Random", [random_of](const Shape& shape, Scalar_ s) { return random_of(cpu(), shape, s); }, py::arg("shape"),
+        py::arg("scalar") = Scalar_::Real);
   m.def("Weight",
         [](const DevPtr& dev, const Shape& shape, Scalar_ s) -> py::object {
           switch (s) {

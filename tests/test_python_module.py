@@ -69,6 +69,151 @@ def test_nodes_on_cpu_compute_or_fail_loudly(ginn):
         ginn.Variance(x).forward()
 
 
+def test_devices_as_in_the_reference(ginn):
+    """ginn-py/test/test_dev.py:29-106 on the CPU devices: a fresh Cpu() and the cpu() singleton are different
+    devices with equal ids, an arena counts exactly the bytes of what lives on it (tensors of every scalar, the
+    value and the empty gradient of a data node, the result of a node), clear() empties it."""
+    d1 = ginn.Cpu()
+    assert d1 == d1 and d1.id == d1.id and d1.precedence == 0
+    d2 = ginn.PreallocCpu(100)
+    assert d2.size == 100 and d1.id == d2.id and d2.precedence == 1 and d2.used == 0
+    t = ginn.RealTensor(d2, [3], [1, 2, 3])
+    assert d2.used == 12 and t.list() == [1, 2, 3]
+    d2.clear()
+    assert d2.used == 0
+    t2, t3 = ginn.RealTensor(ginn.cpu(), [], [0]), ginn.RealTensor(ginn.cpu(), [], [0])
+    assert t2.dev == t3.dev and t2.dev != d1
+    assert ginn.cpu().kind == ginn.DeviceType.CPU and repr(d1.id) == "<DeviceId with kind: CPU, idx: 0>"
+    for scalar, size in [(ginn.Real, 4), (ginn.Half, 2), (ginn.BFloat16, 2), (ginn.Int, 4), (ginn.Bool, 1)]:
+        dev = ginn.PreallocCpu(100)
+        t1 = ginn.Tensor(ginn.cpu(), [2, 3], scalar=scalar)
+        assert dev.used == 0
+        t2 = ginn.Tensor(dev, [1, 2], scalar=scalar)
+        assert dev.used == t2.size * size
+        ginn.Tensor(dev, scalar=scalar)
+        assert dev.used == t2.size * size
+        t4 = t2.copy_to(dev)
+        assert dev.used == 2 * t2.size * size and t4.dev == dev
+        t1.maybe_copy_to(dev)
+        t1.move_to(dev)
+        assert dev.used == (2 * t2.size + t1.size) * size
+        t2.move_to(dev)  # already there
+        assert dev.used == (2 * t2.size + t1.size) * size
+    for Data, size in [(ginn.RealData, 4), (ginn.HalfData, 2)]:
+        dev = ginn.PreallocCpu(100)
+        x, y = Data(ginn.cpu(), [1, 2]), Data(ginn.cpu(), [1, 2])
+        x.has_grad = False
+        x.move_to(dev)
+        assert dev.used == x.size * size
+        y.move_to(dev)  # value and the (empty) gradient
+        assert dev.used == 2 * x.size * size
+        z = ginn.Add(x, y)
+        g = ginn.Graph(z)
+        assert dev.used == 2 * x.size * size
+        g.forward()
+        assert dev.used == 3 * x.size * size
+
+
+def test_tensor_constructors_casts_and_views(ginn):
+    """ginn-py/test/test_tensor.py: the constructor forms (:22-55), casts (:58-82), values and equality
+    (:85-112), m() / v() as views that write through (:115-127), resizing through `shape` (:130-151)."""
+    kinds = [(ginn.RealTensor, ginn.Real), (ginn.HalfTensor, ginn.Half), (ginn.IntTensor, ginn.Int),
+             (ginn.BoolTensor, ginn.Bool), (ginn.BFloat16Tensor, ginn.BFloat16)]
+    for cls, scalar in kinds:
+        for t in (cls(), cls([2]), cls(ginn.cpu()), cls(ginn.cpu(), [2]), ginn.Tensor(scalar=scalar),
+                  ginn.Tensor(scalar=scalar, shape=[2]), ginn.Tensor(device=ginn.cpu(), scalar=scalar),
+                  ginn.Tensor(shape=[2], scalar=scalar, device=ginn.cpu())):
+            assert t.scalar == scalar and all(t.scalar != other for _, other in kinds if other != scalar)
+        t = cls(ginn.cpu())
+        t.set([[1, 2, 3], [4, 5, 6]])
+        assert t.real() == t.cast(ginn.Real) and t.int() == t.cast(ginn.Int)
+        assert t.half() == t.cast(ginn.Half) and t.bool() == t.cast(ginn.Bool)
+        assert t.cast(ginn.Real).scalar == ginn.Real and t.int().scalar == ginn.Int
+    assert ginn.Tensor().scalar == ginn.Real and ginn.Tensor([2]).shape == [2]
+    a, c, d = ginn.RealTensor(), ginn.RealTensor(), ginn.RealTensor()
+    a.set([1, 2, 3])
+    c.set([[1, 2, 3], [4, 5, 6]])
+    d.set([[1, 2, 3], [4, 5, 6]])
+    assert a.shape == [3] and c.shape == [2, 3] and a == a and a != c and c == d
+    assert a.list() == [1, 2, 3] and c.list() == [1, 4, 2, 5, 3, 6]
+    c.set_zero()
+    assert c.list() == [0] * 6
+    c.set_ones()
+    assert c.list() == [1] * 6
+    c.set_random()
+    vals = c.list()
+    assert all(-1 <= x <= 1 for x in vals) and all(x != y for x, y in zip(vals[:-1], vals[1:]))
+    a = ginn.RealTensor([2, 3], [1, 2, 3, 4, 5, 6])
+    np.testing.assert_array_equal(a.v(), np.array([1, 2, 3, 4, 5, 6], np.float32))
+    np.testing.assert_array_equal(a.m(), np.array([[1, 3, 5], [2, 4, 6]], np.float32))
+    v = a.v()
+    v[3] = -4
+    assert a.list() == [1, 2, 3, -4, 5, 6]
+    m = a.m()
+    m[0, 1] = -3
+    assert a.list() == [1, 2, -3, -4, 5, 6]
+    vals = [1, 2, 3, 4, 5, 6]
+    a = ginn.RealTensor(ginn.cpu(), [2, 1, 3], vals)
+    for shape in ([6], [3, 2]):
+        a.shape = shape
+        assert a.size == 6 and a.shape == shape and a.list() == vals
+    for shape in ([4], [2, 2]):
+        a.shape = shape
+        assert a.size == 4 and a.shape == shape
+    assert ginn.RealTensor([1], [2.5]).item() == 2.5
+
+
+def test_keyword_forms_of_the_reference(ginn):
+    """The argument names ginn-py gives its factories (ginn-py/node-py.cu.cpp:181-220, node/layout-py.cu.cpp,
+    node/common-py.cu.cpp, node/weight-py.cu.cpp), as its tests call them (ginn-py/test/test_nodes.py:57, 76, 100,
+    177, 216, 382, 942)."""
+    dev = ginn.cpu()
+    assert ginn.Random(dev, [3, 2, 1], scalar=ginn.Real).shape == [3, 2, 1]
+    assert ginn.Random(device=dev, shape=[2, 2], scalar=ginn.Half).value.scalar == ginn.Half
+    assert ginn.Random(shape=[4]).shape == [4]
+    v = ginn.Values(values=[1, 2, 3, 4], dev=dev)
+    assert v.value.list() == [1, 2, 3, 4] and ginn.Values(values=[[1, 2], [3, 4]]).shape == [2, 2]
+    W = ginn.Values(dev, [[1, 2, 3, 4, 5, 6]])
+    r = ginn.Reshape(W, shape=[3, 2])
+    r.forward()
+    assert r.shape == [3, 2]
+    x = ginn.Values(dev, [[1, 2], [3, 4], [5, 6], [7, 8]])
+    sl = ginn.Slice(x, offsets=[0, 1], sizes=[4, 1])
+    ginn.Graph(sl).forward()
+    assert sl.value.list() == [2, 4, 6, 8]
+    ch = ginn.Chip(x, offset=2, dim=0)
+    ginn.Graph(ch).forward()
+    assert ch.value.list() == [5, 6]
+    w = ginn.Weight(scalar=ginn.Real, device=dev, shape=[2, 3])
+    assert w.shape == [2, 3] and w.copy(mode=ginn.Copy.Tied).shape == [2, 3]
+    assert ginn.Data(dev, scalar=ginn.Half).value.scalar == ginn.Half
+    assert ginn.Data([2, 3], scalar=ginn.Int).shape == [2, 3]
+    assert ginn.Data(device=dev, shape=[2], scalar=ginn.Bool).value.scalar == ginn.Bool
+    a, b, c = (ginn.Values(dev, [[1.0, 2.0]]) for _ in range(3))
+    cpa = ginn.CwiseProdAdd(a, multiplicand=b, addend=c, multiplicand_bias=1.0)
+    ginn.Graph(cpa).forward()
+    assert cpa.value.list() == [3.0, 8.0]
+    mask = ginn.Random(device=dev, shape=[2, 2]) * 0.5 + 1.0  # ginn-py/test/test_nodes.py check_grad's mask
+    ginn.Graph(mask).forward()
+    assert all(0.5 <= m <= 1.5 for m in mask.value.list())
+
+
+def test_dim_nodes(ginn):
+    """ginn-py/test/test_nodes.py:53-70 and the broadcasts that take a Dim (:334-335, 357-358), on cpu() where
+    the broadcast is a view (extent 1) or refused loudly (a copy needs the device)."""
+    x = ginn.Data(ginn.cpu(), [3, 2, 1])
+    dims = [ginn.Dim(x, i) for i in range(3)]
+    for d in dims:
+        ginn.Graph(d).forward()
+    assert [d.value for d in dims] == [3, 2, 1]
+    assert ginn.Dim(7).value == 7
+    a = ginn.Values(ginn.cpu(), [[1], [2], [3]])
+    b = ginn.Values(ginn.cpu(), [[0.5, 1.5, 2.5]])
+    same = ginn.ColBroadcast(a, ginn.Dim(b, 0))
+    ginn.Graph(same).forward()
+    assert same.shape == [3, 1] and same.value.list() == [1, 2, 3]
+
+
 @pytest.mark.gpu
 def test_mnist_style_training_loop(ginn):
     from oracle import nodes as N
