@@ -400,6 +400,96 @@ def test_reference_python_cases(ginn, scalar_name):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("scalar_name", ["Real", "Half"])
+def test_reference_python_cases_of_the_other_nodes(ginn, scalar_name):
+    """test_nonlin (:560-606), test_nonlin_extreme (:609-631), test_pick_and_friends (:634-672), test_axis_sum
+    (:735-760), test_reduce (:771-784), test_weight (:940-962) and the Stack errors (:120-140) of
+    ginn-py/test/test_nodes.py, forward, on the device, with the tolerances used there."""
+    scalar = getattr(ginn, scalar_name)
+    dev = ginn.gpu()
+    half = scalar_name == "Half"
+
+    def vals(v):
+        return ginn.Values(dev, v).cast(scalar)
+
+    def check(a, b, eps=1e-6):
+        ginn.Graph(a).forward()
+        ginn.Graph(b).forward()
+        a_, b_ = a.value.maybe_copy_to(ginn.cpu()), b.value.maybe_copy_to(ginn.cpu())
+        assert a_.shape == b_.shape
+        eps = max(eps, 1e-3) if half else eps
+        assert a_.list() == pytest.approx(b_.list(), rel=eps, abs=eps * 1e-1)
+
+    W = vals([[-1, -2, -3], [4, 5, 6]])
+    absW = vals([[1, 2, 3], [4, 5, 6]])
+    check(ginn.Identity(W), W)
+    check(ginn.Tanh(W), vals([[-0.76159415, -0.96402758, -0.99505475], [0.99932929, 0.99990920, 0.99998771]]))
+    check(ginn.Relu(W), vals([[0, 0, 0], [4, 5, 6]]))
+    check(ginn.Sigmoid(W), vals([[0.26894142, 0.11920292, 0.04742587], [0.98201379, 0.99330714, 0.99752737]]))
+    check(ginn.Softmax(W), vals([[0.00669285, 9.11051194e-04, 1.23394576e-04],
+                                 [0.99330715, 9.99088949e-01, 9.99876605e-01]]))
+    check(ginn.Sqrt(ginn.CwiseProd(W, W)), absW)
+    check(ginn.Log(absW), vals([[0, 0.69314718, 1.09861229], [1.38629436, 1.60943791, 1.79175947]]))
+    x = vals([[10000.0], [-10000.0]])
+    x2 = vals([[5.0], [-float("inf")]])
+    check(ginn.Tanh(x), vals([[1], [-1]]))
+    check(ginn.Sigmoid(x) + 1.0, vals([[1], [0]]) + 1.0)
+    check(ginn.Softmax(ginn.Reshape(x, [1, 2])), ginn.Reshape(vals([[1], [1]]), [1, 2]))
+    check(ginn.Softmax(x), vals([[1], [0]]))
+    check(ginn.Softmax(x2), vals([[1], [0]]))
+
+    P = vals([[-0.5, 0.55, -0.45], [1.0, 2.0, -1.0], [0.0, 0.0, 0.0], [0.3, -0.33, 1.3]])
+    p, psm = vals([[0.3, 0.55, -1.0]]), vals([[0.23787436, 0.15987601, 0.06482681]])
+    pnlsm = vals([[1.43601264, 1.8333567, 2.73603603]])
+    il = [3, 0, 1]
+    it = ginn.Values(dev, [3, 0, 1]).cast(ginn.Int)
+    it.has_grad = False
+    for idx in (il, it):
+        check(ginn.Pick(P, idx), p)
+        check(ginn.PickSoftmax(P, idx), psm)
+        check(ginn.Pick(ginn.Softmax(P), idx), psm)
+        check(ginn.PickNegLogSoftmax(P, idx), pnlsm)
+        check(ginn.Pick(-ginn.Log(ginn.Softmax(P)), idx), pnlsm)
+        check(-ginn.Log(ginn.Pick(ginn.Softmax(P), idx)), pnlsm)
+
+    V = vals([[[1, 2, 3], [4, 5, 6]], [[0.1, 0.2, 0.3], [0.4, 0.5, 0.6]]])
+    check(ginn.AxisSum(V, [0]), vals([[1.1, 2.2, 3.3], [4.4, 5.5, 6.6]]))
+    check(ginn.AxisSum(V, [0, 1]), vals([5.5, 7.7, 9.9]))
+    check(ginn.AxisSum(V, [0, 1, 2]), vals(23.1))
+    check(ginn.AxisSum(V, [1]), vals([[5, 7, 9], [0.5, 0.7, 0.9]]))
+    check(ginn.AxisSum(V, [1, 2]), vals([21, 2.1]))
+    check(ginn.AxisSum(V, [2]), vals([[6, 15], [0.6, 1.5]]))
+    check(ginn.AxisSum(V, [0, 2]), vals([6.6, 16.5]))
+    for bad in ([0, 0], [2, 0]):
+        with pytest.raises(RuntimeError):
+            ginn.AxisSum(V, bad)
+    M = vals([[1, 2, 3], [4, 5, 6]])
+    check(ginn.Sum(M), vals(21))
+    check(ginn.Mean(M), vals(3.5))
+    check(ginn.Variance(M), vals(35.0 / 12.0))
+
+    a, b, c, d = (vals([1 + 4 * i, 2 + 4 * i, 3 + 4 * i, 4 + 4 * i]) for i in range(4))
+    e, f = vals([17, 18, 19]), vals([21, 22, 23, 24])
+    for grid in ([[a, b], [c, d], [e, f]], [[a, b], [c, d], [e]], []):
+        with pytest.raises(RuntimeError):
+            ginn.Graph(ginn.Stack(grid)).forward()
+
+    Wt = ginn.Weight(scalar=scalar, device=dev, shape=[2, 3])
+    Wt.set_random()
+    t = Wt.value.copy_to(dev)
+    assert Wt.forwarded
+    Wt.reset_forwarded()
+    assert Wt.forwarded
+    Wt.forward()
+    assert Wt.value == t
+    Wt.reset_grad()
+    W2 = Wt.copy(ginn.Copy.Tied)
+    assert W2.value is Wt.value and W2.grad is not Wt.grad
+    W3 = Wt.copy(ginn.Copy.Deep)
+    assert W3.value == Wt.value and W3.value is not Wt.value and W3.grad is not Wt.grad
+
+
+@pytest.mark.gpu
 def test_int_nodes_through_the_bindings(ginn):
     """The cases of ginn-py/test/test_nodes.py that run on ginn.Int (scalars3: Stack :73-118, test_add :388,
     test_add_scalar :416, test_subtract_scalar :434, test_prod_scalar :459, test_cwise_prod :476, CwiseProdAdd
