@@ -443,7 +443,8 @@ def bench_skinny(h, steps, warmup):
         ms = time_product(h, dt, "NN", m, n, k, steps, warmup)
         by = ESIZE[dt] * (m * k + k * n + m * n)
         out.append({"config": f"{dt} NN {m}x{n}x{k}", "us": round(ms * 1e3, 2), "gbs": round(by / ms / 1e6, 1),
-                    "frac_hbm": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)})
+                    "frac_hbm": round(by / ms / 1e6 / PEAK_HBM_GBS, 4),
+                    "frac_mfma": round(2.0 * m * n * k / ms / 1e9 / PEAK_TFLOPS[dt], 4)})
     return out
 
 
@@ -625,8 +626,10 @@ def other_configs(h, cpu):
         for nn in (1, 16, 64):
             ms = time_product(h, dt, "NN", 4096, nn, 4096, 200, 20)
             by = ESIZE[dt] * (4096 * 4096 + 4096 * nn + 4096 * nn)
+            tf = 2.0 * 4096 * nn * 4096 / ms / 1e9
             skinny[f"{dt}_n{nn}"] = {"us": round(ms * 1e3, 2), "gbs": round(by / ms / 1e6, 1),
-                                     "frac_hbm": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)}
+                                     "frac_hbm": round(by / ms / 1e6 / PEAK_HBM_GBS, 4),
+                                     "frac_mfma": round(tf / PEAK_TFLOPS[dt], 4)}
     out["skinny_m4096_k4096"] = skinny
     squares = {}
     for size, steps in ((4096, 100), (2048, 200)):
