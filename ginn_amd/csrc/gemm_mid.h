@@ -543,7 +543,10 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
     claim_frags(0);
     __builtin_amdgcn_sched_barrier(0);
     multiply(0);
-    __builtin_amdgcn_sched_barrier(0);
+    // fp32: an MFMA keeps the pipe for 64 cycles, so the refills of a set may go out between its MFMAs as their
+    // registers fall free (the compiler places them; the order of the reads among themselves, which the
+    // waits by count rely on, stays).  16 bit: the refills follow the set's MFMAs as a block.
+    if constexpr (!F32IN) __builtin_amdgcn_sched_barrier(0);
     if (more) {
       issue_frags(J0);
       lgkm_wait<kReads>();
@@ -553,7 +556,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(MidParams p) {
     claim_frags(1);
     __builtin_amdgcn_sched_barrier(0);
     multiply(1);
-    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!F32IN) __builtin_amdgcn_sched_barrier(0);
     if (more) issue_frags(J1);
   };
 
