@@ -820,3 +820,147 @@ def test_multi_chain(dev):
     dev.lib.call("ginn_hip_multi_chain", dev.ctx, 0, None, None)
     with pytest.raises(capi.GinnHipError):
         dev.lib.call("ginn_hip_multi_chain", dev.ctx, 3, None, None)
+
+
+def test_multi_chain_overlapping_operands(dev):
+    """Chains whose records read and write overlapping memory in every way a graph can ask for, each checked
+    against the records applied one after the other on the host: the element-wise part of a recurrent cell (a
+    1024-element sum, four slices of it copied, nonlinearities, products, a sum, a result written into a column
+    of a table), lengths that are no multiples of the workgroup, in-place and accumulating records, a record that
+    writes over an earlier record's source, operands that are shifted against each other (a source that overlaps
+    an earlier destination at another offset, or reaches beyond it into what memory held before)."""
+    import struct
+    t = dev.torch
+    rng = np.random.default_rng(17)
+    SUM, PROD, FWD, BWD, FILL = 1, 2, 3, 4, 0
+    arena = t.zeros(1 << 20, dtype=t.float32, device="cuda")  # one allocation: every offset below is in floats
+    base_ptr = arena.data_ptr()
+    assert base_ptr % 1024 == 0
+    initial = np.zeros(1 << 20, np.float32)
+    cursor = [0]
+    records, ranges = [], []
+
+    def alloc(n, shift=0, init=None):
+        off = (cursor[0] + 255) // 256 * 256 + shift  # on the grid of 256 floats, plus `shift` floats
+        cursor[0] = off + n + 256
+        if init is not None:
+            initial[off:off + n] = init
+        return off
+
+    def rec(kind, act, acc, value, stage, n, dst, *srcs):
+        srcs = list(srcs) + [None] * (3 - len(srcs))
+        ptrs = [0 if o is None else base_ptr + 4 * o for o in srcs]
+        records.append((struct.pack("<iiiifiQQQQQ", capi.F32, kind, act, acc, value, stage, n, base_ptr + 4 * dst, *ptrs),
+                        (kind, act, acc, value, n, dst, srcs)))
+
+    def begin():
+        return len(records)
+
+    def end(first):
+        ranges.append((first, len(records) - first))
+
+    def rnd(n):
+        return rng.standard_normal(n).astype(np.float32)
+
+    # 1. the element-wise part of an LSTM step, several chains of it
+    for _ in range(6):
+        H = 256
+        prod, bias, c_prev = alloc(4 * H, init=rnd(4 * H)), alloc(4 * H, init=rnd(4 * H)), alloc(H, init=rnd(H))
+        z = alloc(4 * H)
+        gates = [alloc(H) for _ in range(4)]
+        acts = [alloc(H) for _ in range(4)]
+        fc, ig, c, tc, h = (alloc(H) for _ in range(5))
+        out = alloc(H, shift=128)  # a column of a table: 512 bytes off the grid
+        f0 = begin()
+        rec(SUM, 0, 0, 0.0, 0, 4 * H, z, prod, bias)
+        for q in range(4):
+            rec(SUM, 0, 0, 0.0, 1, H, gates[q], z + H * [3, 1, 0, 2][q])
+        for q in range(4):
+            rec(FWD, N.TANH if q == 3 else N.SIGMOID, 0, 0.0, 2, H, acts[q], gates[q])
+        rec(PROD, 0, 0, 0.0, 3, H, fc, acts[1], c_prev)
+        rec(PROD, 0, 0, 0.0, 3, H, ig, acts[2], acts[3])
+        rec(SUM, 0, 0, 0.0, 4, H, c, fc, ig)
+        rec(FWD, N.TANH, 0, 0.0, 5, H, tc, c)
+        rec(PROD, 0, 0, 0.0, 6, H, h, acts[0], tc)
+        rec(SUM, 0, 0, 0.0, 7, H, out, h)
+        end(f0)
+    # 2. lengths that fill no block, in-place and accumulating records, the gradient of a nonlinearity
+    for n in (4, 200, 255, 257, 1000, 1024):
+        x, y, g = alloc(n, init=rnd(n)), alloc(n), alloc(n, init=rnd(n))
+        acc = alloc(n, init=rnd(n))
+        f0 = begin()
+        rec(FWD, N.TANH, 0, 0.0, 0, n, y, x)
+        rec(BWD, N.TANH, 0, 0.0, 1, n, g, g, x, y)      # in place: g = g * (1 - y^2)
+        rec(SUM, 0, 1, 0.0, 2, n, acc, g)                # acc += g
+        rec(PROD, 0, 1, 0.0, 3, n, acc, acc, y)          # acc += acc * y (reads what it adds to)
+        rec(FILL, 0, 0, 2.5, 4, n, x)                    # writes over a source of stage 0
+        rec(SUM, 0, 0, 0.0, 5, n, y, x, acc)             # y = 2.5 + acc, over an earlier destination
+        end(f0)
+    # 3. all operands at the same offset from the grid
+    for shift in (1, 77):
+        n = 300
+        x, y, w = alloc(n, shift, rnd(n)), alloc(n, shift), alloc(n, shift)
+        f0 = begin()
+        rec(FWD, N.SIGMOID, 0, 0.0, 0, n, y, x)
+        rec(PROD, 0, 0, 0.0, 1, n, w, y, x)
+        rec(SUM, 0, 0, 0.0, 2, n, y, w, y)
+        end(f0)
+    # 4. a source overlapping an earlier destination at another offset: values pass between threads
+    n = 256
+    x, y = alloc(n + 8, init=rnd(n + 8)), alloc(n + 8, init=rnd(n + 8))
+    w = alloc(n)
+    f0 = begin()
+    rec(FWD, N.TANH, 0, 0.0, 0, n, y, x)
+    rec(SUM, 0, 0, 0.0, 1, n, w, y + 4, x + 4)  # reads y shifted by four elements
+    end(f0)
+    # 5. a source that reaches beyond the destination it overlaps
+    x, y, w = alloc(256, init=rnd(256)), alloc(256, init=rnd(256)), alloc(256)
+    f0 = begin()
+    rec(FWD, N.RELU, 0, 0.0, 0, 200, y, x)
+    rec(SUM, 0, 0, 0.0, 1, 256, w, y, x)  # elements 200 .. 255 of y are what memory held
+    end(f0)
+    # 6. a record that writes over the source of an earlier one at another offset
+    x, y = alloc(512, init=rnd(512)), alloc(256)
+    f0 = begin()
+    rec(FWD, N.TANH, 0, 0.0, 0, 256, y, x)
+    rec(FILL, 0, 0, -1.0, 1, 256, x + 128)
+    rec(SUM, 0, 0, 0.0, 2, 256, y, y, x)
+    end(f0)
+    # the records applied one after the other on the host, in double precision with fp32 results
+    def act(code, v):
+        return {N.TANH: np.tanh, N.SIGMOID: lambda u: 1 / (1 + np.exp(-u)), N.RELU: lambda u: np.maximum(u, 0)}[code](v)
+
+    assert cursor[0] < initial.size
+    host = initial.copy()
+    for _, (kind, a, acc, value, n, dst, srcs) in records:
+        ins = [None if o is None else host[o:o + n].astype(np.float64) for o in srcs]
+        if kind == FILL:
+            v = np.full(n, value)
+        elif kind == SUM:
+            v = sum(i for i in ins if i is not None)
+        elif kind == PROD:
+            v = ins[0] * ins[1]
+        elif kind == FWD:
+            v = act(a, ins[0])
+        else:
+            assert a == N.TANH
+            v = ins[0] * (1 - ins[2] ** 2)
+        if acc:
+            v = v + host[dst:dst + n]
+        host[dst:dst + n] = v.astype(np.float32)
+
+    table = t.frombuffer(bytearray(b"".join(r for r, _ in records)), dtype=t.uint8).to("cuda")
+    rtable = t.frombuffer(bytearray(b"".join(struct.pack("<II", f, c) for f, c in ranges)), dtype=t.uint8).to("cuda")
+    touched = np.zeros(initial.size, bool)
+    for _, (_, _, _, _, n, dst, _) in records:
+        touched[dst:dst + n] = True
+    for _ in range(2):  # twice from the same start
+        arena.copy_(t.from_numpy(initial))
+        dev.lib.call("ginn_hip_multi_chain", dev.ctx, len(ranges), c_void_p(rtable.data_ptr()), c_void_p(table.data_ptr()))
+        dev.sync()
+        got = arena.cpu().numpy()
+        for first, count in ranges:
+            for _, (kind, a, acc, value, n, dst, srcs) in records[first:first + count]:
+                np.testing.assert_allclose(got[dst:dst + n], host[dst:dst + n], rtol=3e-5, atol=3e-6,
+                                           err_msg=f"chain at record {first}, destination {dst}, n {n}")
+        np.testing.assert_array_equal(got[~touched], initial[~touched])  # nothing else was written
